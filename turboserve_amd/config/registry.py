@@ -1,4 +1,5 @@
-"""One registry from an architecture's name (``config.json``'s ``architectures[0]``) to its
+"""One registry from an architecture's name (``config.json``'s ``architectures[0]``, or its
+``architecture`` where the file names the design that way) to its
 configuration class and its plan builder.
 
 The reference keeps only a dict of names (src/turboserve/engine/model/model_config.py:41-44)
@@ -35,7 +36,7 @@ def architecture_of(data: Mapping[str, Any]) -> Architecture:
     """The registered architecture a ``config.json`` mapping names."""
     _ensure_builtin()
     names = data.get("architectures") or []
-    name = str(names[0]) if names else ""
+    name = str(names[0]) if names else str(data.get("architecture") or "")
     if name not in ARCHITECTURES:
         raise UnsupportedModelError(
             f"architecture {name or '<missing>'!r} is not implemented; supported: {sorted(ARCHITECTURES)}"
@@ -53,3 +54,8 @@ def _ensure_builtin() -> None:
         from turboserve_amd.models.qwen2 import qwen2_plan
 
         register_architecture("Qwen2ForCausalLM", Qwen2Config.from_dict, qwen2_plan)
+    if "Sisisun" not in ARCHITECTURES:
+        from turboserve_amd.config.sisisun_config import SisisunConfig
+        from turboserve_amd.models.sisisun import sisisun_plan
+
+        register_architecture("Sisisun", SisisunConfig.from_dict, sisisun_plan)

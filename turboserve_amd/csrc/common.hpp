@@ -123,4 +123,21 @@ __device__ __forceinline__ ts_u32x4 load_once16(const void* at) {
   return __builtin_nontemporal_load(reinterpret_cast<const ts_u32x4*>(at));
 }
 
+// The gated unit of a feed-forward: with g' = min(g, limit) and u' = clamp(u, -limit, limit) where
+// limit > 0 (else g' = g, u' = u), g' * sigmoid(steepness * g') * (u' + up_shift).  silu(g) * u is
+// {1, 0, 0}.
+struct GluRule {
+  float steepness;
+  float limit;
+  float up_shift;
+};
+
+__device__ __forceinline__ float gated_unit(float g, float u, GluRule rule) {
+  if (rule.limit > 0.f) {
+    g = fminf(g, rule.limit);
+    u = fminf(fmaxf(u, -rule.limit), rule.limit);
+  }
+  return g / (1.f + expf(-(rule.steepness * g))) * (u + rule.up_shift);
+}
+
 static inline int ts_launch_status() { return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH; }

@@ -48,9 +48,17 @@ extern "C" int ts_embed(void* residual, const void* table, const int* ids, int t
 // kernel reads rows[i] and writes y[i] only (residual untouched): the final norm at the wanted
 // positions.
 // ---------------------------------------------------------------------------------------------
+// The gain: `one_rounding == 0` is the rule above, w * round_T(n); otherwise the whole norm is
+// 32-bit arithmetic with one rounding at the end, round_T(n * (gain_offset + w)) (a gain stored
+// around zero has gain_offset 1).
+template <typename T>
+__device__ __forceinline__ float with_gain(float normalised, float gain, float gain_offset, int one_rounding) {
+  return one_rounding ? normalised * (gain_offset + gain) : gain * round_to<T>(normalised);
+}
+
 template <typename T>
 __global__ void rmsnorm_kernel(T* __restrict__ y, const T* __restrict__ x, const T* __restrict__ w,
-                               float eps, int hidden) {
+                               float eps, int hidden, float gain_offset, int one_rounding) {
   __shared__ float scratch[16];
   const size_t base = (size_t)blockIdx.x * hidden;
   float ss = 0.f;
@@ -61,8 +69,7 @@ __global__ void rmsnorm_kernel(T* __restrict__ y, const T* __restrict__ x, const
   ss = block_sum(ss, scratch);
   const float rstd = rsqrtf(ss / (float)hidden + eps);
   for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
-    const float n = round_to<T>(to_float(x[base + i]) * rstd);
-    y[base + i] = from_float<T>(to_float(w[i]) * n);
+    y[base + i] = from_float<T>(with_gain<T>(to_float(x[base + i]) * rstd, to_float(w[i]), gain_offset, one_rounding));
   }
 }
 
@@ -91,7 +98,7 @@ template <typename T, typename P>
 __global__ void add_rmsnorm_kernel(T* __restrict__ y, float* __restrict__ residual,
                                    const P* __restrict__ pending, int splits, size_t split_stride,
                                    const T* __restrict__ w, const int* __restrict__ rows, float eps,
-                                   int hidden) {
+                                   int hidden, float gain_offset, int one_rounding) {
   __shared__ float scratch[16];
   const int src = rows ? rows[blockIdx.x] : blockIdx.x;
   const size_t in_base = (size_t)src * hidden;
@@ -110,20 +117,19 @@ __global__ void add_rmsnorm_kernel(T* __restrict__ y, float* __restrict__ residu
   for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
     float s = residual[in_base + i];
     if (rows && pending) s = add_splits(pending + in_base + i, splits, split_stride, s);
-    const float n = round_to<T>(s * rstd);
-    y[out_base + i] = from_float<T>(to_float(w[i]) * n);
+    y[out_base + i] = from_float<T>(with_gain<T>(s * rstd, to_float(w[i]), gain_offset, one_rounding));
   }
 }
 
 extern "C" int ts_rmsnorm(void* y, const void* x, const void* w, float eps, int tokens, int hidden,
-                          int dtype, hipStream_t stream) {
+                          float gain_offset, int one_rounding, int dtype, hipStream_t stream) {
   if (tokens == 0) return TS_OK;
   if (!y || !x || !w || hidden < 1) return TS_ERR_ARG;
   dim3 grid(tokens), block(hidden <= 1024 ? 256 : 1024);
   if (dtype == TS_F32)
-    hipLaunchKernelGGL(rmsnorm_kernel<float>, grid, block, 0, stream, (float*)y, (const float*)x, (const float*)w, eps, hidden);
+    hipLaunchKernelGGL(rmsnorm_kernel<float>, grid, block, 0, stream, (float*)y, (const float*)x, (const float*)w, eps, hidden, gain_offset, one_rounding);
   else if (dtype == TS_BF16)
-    hipLaunchKernelGGL(rmsnorm_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)y, (const bf16_t*)x, (const bf16_t*)w, eps, hidden);
+    hipLaunchKernelGGL(rmsnorm_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)y, (const bf16_t*)x, (const bf16_t*)w, eps, hidden, gain_offset, one_rounding);
   else
     return TS_ERR_DTYPE;
   return ts_launch_status();
@@ -201,7 +207,7 @@ template <typename T, typename P>
 __global__ void add_rmsnorm_vec4_kernel(T* __restrict__ y, float* __restrict__ residual,
                                         const P* __restrict__ pending, int splits, size_t split_stride,
                                         const T* __restrict__ w, const int* __restrict__ rows, float eps,
-                                        int hidden) {
+                                        int hidden, float gain_offset, int one_rounding) {
   __shared__ float scratch[16];
   const int src = rows ? rows[blockIdx.x] : blockIdx.x;
   const size_t in_base = (size_t)src * hidden;
@@ -231,7 +237,7 @@ __global__ void add_rmsnorm_vec4_kernel(T* __restrict__ y, float* __restrict__ r
     if (qd < quads) {
       float o[4];
 #pragma unroll
-      for (int e = 0; e < 4; ++e) o[e] = g[it][e] * round_to<T>(s[it][e] * rstd);
+      for (int e = 0; e < 4; ++e) o[e] = with_gain<T>(s[it][e] * rstd, g[it][e], gain_offset, one_rounding);
       Vec4Of<T>::store(y + out_base + 4 * qd, o);
     }
   }
@@ -240,18 +246,19 @@ __global__ void add_rmsnorm_vec4_kernel(T* __restrict__ y, float* __restrict__ r
 template <typename T, typename P>
 static void launch_add_rmsnorm(void* y, float* residual, const void* pending, int splits, long split_stride,
                                const void* w, const int* rows, float eps, int out_rows, int hidden,
-                               hipStream_t stream) {
+                               float gain_offset, int one_rounding, hipStream_t stream) {
   // Few rows (decode): one large block per row; many rows (prefill): just enough threads.
   int threads = out_rows <= 256 ? 1024 : 256;
   const int need = (hidden / 4 + NORM_ITEMS - 1) / NORM_ITEMS;
   if (threads < need) threads = ((need + 63) / 64) * 64;
   if (hidden % 4 == 0 && threads <= 1024) {
     hipLaunchKernelGGL((add_rmsnorm_vec4_kernel<T, P>), dim3(out_rows), dim3(threads), 0, stream, (T*)y, residual,
-                       (const P*)pending, splits, (size_t)split_stride, (const T*)w, rows, eps, hidden);
+                       (const P*)pending, splits, (size_t)split_stride, (const T*)w, rows, eps, hidden, gain_offset,
+                       one_rounding);
   } else {
     hipLaunchKernelGGL((add_rmsnorm_kernel<T, P>), dim3(out_rows), dim3(hidden <= 1024 ? 256 : 1024), 0, stream,
                        (T*)y, residual, (const P*)pending, splits, (size_t)split_stride, (const T*)w, rows, eps,
-                       hidden);
+                       hidden, gain_offset, one_rounding);
   }
 }
 
@@ -259,29 +266,30 @@ static void launch_add_rmsnorm(void* y, float* residual, const void* pending, in
 // pending_f32 != 0: `pending` holds `splits` 32-bit partial sums, `split_stride` elements apart.
 extern "C" int ts_add_rmsnorm(void* y, float* residual, const void* pending, int pending_f32, int splits,
                               long split_stride, const void* w, const int* rows, float eps, int out_rows,
-                              int hidden, int dtype, hipStream_t stream) {
+                              int hidden, float gain_offset, int one_rounding, int dtype, hipStream_t stream) {
   if (out_rows == 0) return TS_OK;
   if (!y || !residual || !w || hidden < 1 || splits < 1) return TS_ERR_ARG;
   if (dtype == TS_F32)
-    launch_add_rmsnorm<float, float>(y, residual, pending, splits, split_stride, w, rows, eps, out_rows, hidden, stream);
+    launch_add_rmsnorm<float, float>(y, residual, pending, splits, split_stride, w, rows, eps, out_rows, hidden, gain_offset, one_rounding, stream);
   else if (dtype == TS_BF16 && pending_f32)
-    launch_add_rmsnorm<bf16_t, float>(y, residual, pending, splits, split_stride, w, rows, eps, out_rows, hidden, stream);
+    launch_add_rmsnorm<bf16_t, float>(y, residual, pending, splits, split_stride, w, rows, eps, out_rows, hidden, gain_offset, one_rounding, stream);
   else if (dtype == TS_BF16)
-    launch_add_rmsnorm<bf16_t, bf16_t>(y, residual, pending, splits, split_stride, w, rows, eps, out_rows, hidden, stream);
+    launch_add_rmsnorm<bf16_t, bf16_t>(y, residual, pending, splits, split_stride, w, rows, eps, out_rows, hidden, gain_offset, one_rounding, stream);
   else
     return TS_ERR_DTYPE;
   return ts_launch_status();
 }
 
 // ---------------------------------------------------------------------------------------------
-// SwiGLU over the fused gate|up projection [T, 2 I]: out[t, i] = silu(gate[t, i]) * up[t, i], with
+// Gated unit over the fused gate|up projection [T, 2 I]: out[t, i] = gated_unit(gate[t, i], up[t, i])
+// (common.hpp; silu(gate) * up is the rule {1, 0, 0}), with
 // gate in the first I columns and up in the last (paired == 0), or alternating: gate i in column
 // 2 i, up i in column 2 i + 1 (paired != 0).
 // ---------------------------------------------------------------------------------------------
 // P: type of the projection output: T, or float for `splits` partial sums to be added up.
 template <typename T, typename P>
 __global__ void swiglu_kernel(T* __restrict__ out, const P* __restrict__ gate_up, int splits,
-                              size_t split_stride, int inter, size_t total, int paired) {
+                              size_t split_stride, int inter, size_t total, int paired, GluRule rule) {
   const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= total) return;
   const size_t t = idx / inter;
@@ -290,14 +298,13 @@ __global__ void swiglu_kernel(T* __restrict__ out, const P* __restrict__ gate_up
   const size_t up_at = paired ? gate_at + 1 : gate_at + inter;
   const float g = add_splits(gate_up + gate_at, splits, split_stride, 0.f);
   const float u = add_splits(gate_up + up_at, splits, split_stride, 0.f);
-  const float act = g / (1.f + expf(-g));
-  out[idx] = from_float<T>(act * u);
+  out[idx] = from_float<T>(gated_unit(g, u, rule));
 }
 
 // Four outputs per thread with 8- or 16-byte loads: for I a multiple of 4.
 template <typename T, typename P>
 __global__ void swiglu_vec4_kernel(T* __restrict__ out, const P* __restrict__ gate_up, int splits,
-                                   size_t split_stride, int inter, size_t quads, int paired) {
+                                   size_t split_stride, int inter, size_t quads, int paired, GluRule rule) {
   const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= quads) return;
   const int per_row = inter / 4;
@@ -321,7 +328,7 @@ __global__ void swiglu_vec4_kernel(T* __restrict__ out, const P* __restrict__ ga
   }
   float o[4];
 #pragma unroll
-  for (int e = 0; e < 4; ++e) o[e] = g[e] / (1.f + expf(-g[e])) * u[e];
+  for (int e = 0; e < 4; ++e) o[e] = gated_unit(g[e], u[e], rule);
   Vec4Of<T>::store(out + t * inter + i, o);
 }
 
@@ -329,7 +336,7 @@ __global__ void swiglu_vec4_kernel(T* __restrict__ out, const P* __restrict__ ga
 // multiple of 8 (the many-row case: a product of the library's, then this).  The same arithmetic
 // per element as above.
 __global__ void swiglu_bf16x8_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ gate_up, int inter,
-                                     size_t octets, int paired) {
+                                     size_t octets, int paired, GluRule rule) {
   const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= octets) return;
   const int per_row = inter / 8;
@@ -353,7 +360,7 @@ __global__ void swiglu_bf16x8_kernel(bf16_t* __restrict__ out, const bf16_t* __r
   }
   float o[8];
 #pragma unroll
-  for (int e = 0; e < 8; ++e) o[e] = g[e] / (1.f + expf(-g[e])) * u[e];
+  for (int e = 0; e < 8; ++e) o[e] = gated_unit(g[e], u[e], rule);
   uint32_t w[4];
 #pragma unroll
   for (int e = 0; e < 4; ++e)
@@ -363,32 +370,34 @@ __global__ void swiglu_bf16x8_kernel(bf16_t* __restrict__ out, const bf16_t* __r
 
 template <typename T, typename P>
 static void launch_swiglu(void* out, const void* gate_up, int splits, long split_stride, int tokens, int inter,
-                          int paired, hipStream_t stream) {
+                          int paired, GluRule rule, hipStream_t stream) {
   if (std::is_same<T, bf16_t>::value && std::is_same<P, bf16_t>::value && splits == 1 && inter % 8 == 0) {
     const size_t octets = (size_t)tokens * (inter / 8);
     hipLaunchKernelGGL(swiglu_bf16x8_kernel, dim3((unsigned)((octets + 255) / 256)), dim3(256), 0, stream,
-                       (bf16_t*)out, (const bf16_t*)gate_up, inter, octets, paired);
+                       (bf16_t*)out, (const bf16_t*)gate_up, inter, octets, paired, rule);
   } else if (inter % 4 == 0) {
     const size_t quads = (size_t)tokens * (inter / 4);
     hipLaunchKernelGGL((swiglu_vec4_kernel<T, P>), dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, stream,
-                       (T*)out, (const P*)gate_up, splits, (size_t)split_stride, inter, quads, paired);
+                       (T*)out, (const P*)gate_up, splits, (size_t)split_stride, inter, quads, paired, rule);
   } else {
     const size_t total = (size_t)tokens * inter;
     hipLaunchKernelGGL((swiglu_kernel<T, P>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, (T*)out,
-                       (const P*)gate_up, splits, (size_t)split_stride, inter, total, paired);
+                       (const P*)gate_up, splits, (size_t)split_stride, inter, total, paired, rule);
   }
 }
 
 extern "C" int ts_swiglu(void* out, const void* gate_up, int in_f32, int splits, long split_stride,
-                         int tokens, int inter, int paired, int dtype, hipStream_t stream) {
+                         int tokens, int inter, int paired, float steepness, float limit, float up_shift,
+                         int dtype, hipStream_t stream) {
   if (tokens == 0) return TS_OK;
   if (!out || !gate_up || inter < 1 || splits < 1) return TS_ERR_ARG;
+  const GluRule rule = {steepness, limit, up_shift};
   if (dtype == TS_F32)
-    launch_swiglu<float, float>(out, gate_up, splits, split_stride, tokens, inter, paired, stream);
+    launch_swiglu<float, float>(out, gate_up, splits, split_stride, tokens, inter, paired, rule, stream);
   else if (dtype == TS_BF16 && in_f32)
-    launch_swiglu<bf16_t, float>(out, gate_up, splits, split_stride, tokens, inter, paired, stream);
+    launch_swiglu<bf16_t, float>(out, gate_up, splits, split_stride, tokens, inter, paired, rule, stream);
   else if (dtype == TS_BF16)
-    launch_swiglu<bf16_t, bf16_t>(out, gate_up, splits, split_stride, tokens, inter, paired, stream);
+    launch_swiglu<bf16_t, bf16_t>(out, gate_up, splits, split_stride, tokens, inter, paired, rule, stream);
   else
     return TS_ERR_DTYPE;
   return ts_launch_status();
@@ -627,5 +636,66 @@ extern "C" int ts_patch_tokens(int* token_ids, const int* patch, const int* sour
   if (!token_ids || !patch || !source || n < 0 || sources < 1) return TS_ERR_ARG;
   hipLaunchKernelGGL(patch_tokens_kernel, dim3((n + 255) / 256), dim3(256), 0, stream, token_ids, patch, source, n,
                      sources);
+  return ts_launch_status();
+}
+
+// ---------------------------------------------------------------------------------------------
+// embedding with a position vector: residual[t, :] = float(table[ids[t], :]) + at[positions[t], :]
+// (`at` is 32-bit, [capacity, hidden]; the host keeps positions below its capacity).
+// ---------------------------------------------------------------------------------------------
+template <typename T>
+__global__ void embed_positions_kernel(float* __restrict__ residual, const T* __restrict__ table,
+                                       const int* __restrict__ ids, const int* __restrict__ positions,
+                                       const float* __restrict__ at, int hidden, int vocab) {
+  const int t = blockIdx.x;
+  const int id = ids[t];
+  const bool valid = id >= 0 && id < vocab;
+  const T* row = table + (size_t)(valid ? id : 0) * hidden;
+  const float* place = at + (size_t)positions[t] * hidden;
+  float* out = residual + (size_t)t * hidden;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x)
+    out[i] = valid ? to_float(row[i]) + place[i] : __uint_as_float(0x7fc00000u);
+}
+
+extern "C" int ts_embed_positions(void* residual, const void* table, const int* ids, const int* positions,
+                                  const float* at, int tokens, int hidden, int vocab, int dtype, hipStream_t stream) {
+  if (tokens == 0) return TS_OK;
+  if (!residual || !table || !ids || !positions || !at || hidden < 1 || vocab < 1) return TS_ERR_ARG;
+  dim3 grid(tokens), block(256);
+  if (dtype == TS_F32)
+    hipLaunchKernelGGL(embed_positions_kernel<float>, grid, block, 0, stream, (float*)residual, (const float*)table, ids, positions, at, hidden, vocab);
+  else if (dtype == TS_BF16)
+    hipLaunchKernelGGL(embed_positions_kernel<bf16_t>, grid, block, 0, stream, (float*)residual, (const bf16_t*)table, ids, positions, at, hidden, vocab);
+  else
+    return TS_ERR_DTYPE;
+  return ts_launch_status();
+}
+
+// ---------------------------------------------------------------------------------------------
+// stream offset: residual[t, :] += origin[t, :] (where given) + offset[:] (where given), 32-bit.
+// ---------------------------------------------------------------------------------------------
+template <typename T>
+__global__ void stream_offset_kernel(float* __restrict__ residual, const float* __restrict__ origin,
+                                     const T* __restrict__ offset, int hidden, size_t total) {
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  float s = residual[idx];
+  if (origin) s += origin[idx];
+  if (offset) s += to_float(offset[idx % hidden]);
+  residual[idx] = s;
+}
+
+extern "C" int ts_stream_offset(float* residual, const float* origin, const void* offset, int tokens, int hidden,
+                                int dtype, hipStream_t stream) {
+  if (tokens == 0) return TS_OK;
+  if (!residual || hidden < 1) return TS_ERR_ARG;
+  const size_t total = (size_t)tokens * hidden;
+  dim3 grid((unsigned)((total + 255) / 256)), block(256);
+  if (dtype == TS_F32)
+    hipLaunchKernelGGL(stream_offset_kernel<float>, grid, block, 0, stream, residual, origin, (const float*)offset, hidden, total);
+  else if (dtype == TS_BF16)
+    hipLaunchKernelGGL(stream_offset_kernel<bf16_t>, grid, block, 0, stream, residual, origin, (const bf16_t*)offset, hidden, total);
+  else
+    return TS_ERR_DTYPE;
   return ts_launch_status();
 }

@@ -1,0 +1,177 @@
+// Per-head normalisation of queries and keys, optional rotary encoding, and the scatter of keys
+// and values into cache pages, for a projection output [T, Hq D + Hkv D + Hkv Dv] (q heads, k
+// heads, v heads; values may have a width of their own).  The projection is of type T, or
+// `splits` 32-bit partial sums that are added up here.
+//
+// A q or k head x of D elements becomes x * rsqrt(mean(x^2) + eps) * (gain_offset + gain[d]) in
+// 32-bit (the gain vector is shared by the heads; a null gain skips the norm), is then rotated by
+// the angles of the token's position where tables are given (pairs (i, i + D/2), as
+// ts_rope_store), and is rounded once.  Queries go to q_out (rows q_stride apart; with a
+// projection of type T this may be the projection itself), keys to key pages [NB, Hkv, BS, D] at
+// slot = page * BS + offset, values to the transposed value pages [NB, Hkv, Dv, BS].  A negative
+// slot or slots == nullptr: nothing is stored for that token.
+#include "common.hpp"
+
+#define HNS_MAX_DIM 512
+#define HNS_WAVES 4
+
+template <typename P>
+__device__ __forceinline__ float sum_of_splits(const P* p, int splits, size_t stride) {
+  float s = to_float(p[0]);
+  for (int i = 1; i < splits; ++i) s += to_float(p[(size_t)i * stride]);
+  return s;
+}
+
+// One wavefront per (token, q or k head).
+template <typename T, typename P>
+__global__ void __launch_bounds__(64 * HNS_WAVES)
+head_norm_store_kernel(T* q_out, long q_stride, const P* proj, int splits, size_t split_stride,
+                       T* __restrict__ k_pages, const T* __restrict__ q_gain, const T* __restrict__ k_gain,
+                       float eps, float gain_offset, const float* __restrict__ cos_table,
+                       const float* __restrict__ sin_table, const int* __restrict__ positions,
+                       const int* __restrict__ slots, int tokens, int heads, int kv_heads, int dim, int vdim,
+                       int block_size) {
+  __shared__ float held[HNS_WAVES][HNS_MAX_DIM];
+  const int wave = threadIdx.x / TS_WAVE, lane = threadIdx.x % TS_WAVE;
+  const int qk_heads = heads + kv_heads;
+  const long item = (long)blockIdx.x * HNS_WAVES + wave;
+  const bool active = item < (long)tokens * qk_heads;
+  const int t = active ? (int)(item / qk_heads) : 0;
+  const int h = active ? (int)(item % qk_heads) : 0;
+  const size_t width = (size_t)qk_heads * dim + (size_t)kv_heads * vdim;
+  const P* row = proj + (size_t)t * width + (size_t)h * dim;
+  const T* gain = h < heads ? q_gain : k_gain;
+  constexpr int PER_LANE = HNS_MAX_DIM / TS_WAVE;
+  float x[PER_LANE];
+  float ss = 0.f;
+#pragma unroll
+  for (int c = 0; c < PER_LANE; ++c) {
+    const int d = lane + c * TS_WAVE;
+    x[c] = (active && d < dim) ? sum_of_splits(row + d, splits, split_stride) : 0.f;
+    ss += x[c] * x[c];
+  }
+  if (gain) {
+    ss = wave_sum(ss);
+    const float r = rsqrtf(ss / (float)dim + eps);
+#pragma unroll
+    for (int c = 0; c < PER_LANE; ++c) {
+      const int d = lane + c * TS_WAVE;
+      if (d < dim) x[c] = x[c] * r * (gain_offset + to_float(gain[d]));
+    }
+  }
+  if (cos_table) {
+#pragma unroll
+    for (int c = 0; c < PER_LANE; ++c) {
+      const int d = lane + c * TS_WAVE;
+      if (d < dim) held[wave][d] = x[c];
+    }
+    __syncthreads();
+    const int half = dim / 2;
+    const size_t at = (size_t)positions[t] * half;
+#pragma unroll
+    for (int c = 0; c < PER_LANE; ++c) {
+      const int d = lane + c * TS_WAVE;
+      if (d < dim) {
+        const int i = d < half ? d : d - half;
+        const float x1 = held[wave][i], x2 = held[wave][i + half];
+        const float cv = cos_table[at + i], sv = sin_table[at + i];
+        x[c] = d < half ? __builtin_fmaf(x1, cv, -(x2 * sv)) : __builtin_fmaf(x2, cv, x1 * sv);
+      }
+    }
+  }
+  if (!active) return;
+  T* dst = nullptr;
+  if (h < heads) {
+    dst = q_out + (size_t)t * q_stride + (size_t)h * dim;
+  } else {
+    const int slot = slots ? slots[t] : -1;
+    if (slot >= 0)
+      dst = k_pages + (((size_t)(slot / block_size) * kv_heads + (h - heads)) * block_size + slot % block_size) * dim;
+  }
+  if (!dst) return;
+#pragma unroll
+  for (int c = 0; c < PER_LANE; ++c) {
+    const int d = lane + c * TS_WAVE;
+    if (d < dim) dst[d] = from_float<T>(x[c]);
+  }
+}
+
+// Values: one block per (group of 8 consecutive tokens, KV head); a thread collects one value
+// dimension of the 8 tokens.  Where the group's slots are 8 consecutive ones that start at a
+// multiple of 8 inside one page, a bfloat16 group leaves as one 16-byte store.
+constexpr int HNS_GROUP = 8;
+
+template <typename T, typename P>
+__global__ void __launch_bounds__(64)
+value_store_kernel(const P* proj, int splits, size_t split_stride, T* __restrict__ v_pages,
+                   const int* __restrict__ slots, int tokens, int heads, int kv_heads, int dim, int vdim,
+                   int block_size) {
+  const int t0 = blockIdx.x * HNS_GROUP;
+  const int kvh = blockIdx.y;
+  const int count = min(HNS_GROUP, tokens - t0);
+  const size_t width = (size_t)(heads + kv_heads) * dim + (size_t)kv_heads * vdim;
+  int slot[HNS_GROUP];
+#pragma unroll
+  for (int j = 0; j < HNS_GROUP; ++j) slot[j] = j < count ? slots[t0 + j] : -1;
+  bool run = sizeof(T) == 2 && count == HNS_GROUP && slot[0] >= 0 && (slot[0] & 7) == 0 && (block_size & 7) == 0;
+#pragma unroll
+  for (int j = 1; j < HNS_GROUP; ++j) run = run && slot[j] == slot[0] + j;
+  const P* column = proj + (size_t)t0 * width + (size_t)(heads + kv_heads) * dim + (size_t)kvh * vdim;
+  for (int d = threadIdx.x; d < vdim; d += blockDim.x) {
+    alignas(16) T v[HNS_GROUP];
+#pragma unroll
+    for (int j = 0; j < HNS_GROUP; ++j)
+      v[j] = from_float<T>(j < count ? sum_of_splits(column + (size_t)j * width + d, splits, split_stride) : 0.f);
+    if (run) {
+      T* dst = v_pages + (((size_t)(slot[0] / block_size) * kv_heads + kvh) * vdim + d) * block_size + slot[0] % block_size;
+      *reinterpret_cast<uint4*>(dst) = *reinterpret_cast<const uint4*>(v);
+    } else {
+#pragma unroll
+      for (int j = 0; j < HNS_GROUP; ++j) {
+        if (slot[j] < 0) continue;
+        v_pages[(((size_t)(slot[j] / block_size) * kv_heads + kvh) * vdim + d) * block_size + slot[j] % block_size] = v[j];
+      }
+    }
+  }
+}
+
+template <typename T, typename P>
+static void launch_head_norm_store(void* q_out, long q_stride, const void* proj, int splits, long split_stride,
+                                   void* k_pages, void* v_pages, const void* q_gain, const void* k_gain, float eps,
+                                   float gain_offset, const float* cos_table, const float* sin_table,
+                                   const int* positions, const int* slots, int tokens, int heads, int kv_heads,
+                                   int dim, int vdim, int block_size, hipStream_t stream) {
+  const long items = (long)tokens * (heads + kv_heads);
+  hipLaunchKernelGGL((head_norm_store_kernel<T, P>), dim3((unsigned)((items + HNS_WAVES - 1) / HNS_WAVES)),
+                     dim3(64 * HNS_WAVES), 0, stream, (T*)q_out, q_stride, (const P*)proj, splits, (size_t)split_stride,
+                     (T*)k_pages, (const T*)q_gain, (const T*)k_gain, eps, gain_offset, cos_table, sin_table, positions,
+                     slots, tokens, heads, kv_heads, dim, vdim, block_size);
+  if (slots)
+    hipLaunchKernelGGL((value_store_kernel<T, P>), dim3((tokens + HNS_GROUP - 1) / HNS_GROUP, kv_heads), dim3(64), 0,
+                       stream, (const P*)proj, splits, (size_t)split_stride, (T*)v_pages, slots, tokens, heads, kv_heads,
+                       dim, vdim, block_size);
+}
+
+extern "C" int ts_head_norm_store(void* q_out, long q_stride, const void* proj, int in_f32, int splits,
+                                  long split_stride, void* k_pages, void* v_pages, const void* q_gain,
+                                  const void* k_gain, float eps, float gain_offset, const float* cos_table,
+                                  const float* sin_table, const int* positions, const int* slots, int tokens,
+                                  int heads, int kv_heads, int dim, int vdim, int block_size, int dtype,
+                                  hipStream_t stream) {
+  if (tokens == 0) return TS_OK;
+  if (!q_out || !proj || !positions || heads < 1 || kv_heads < 1 || dim < 1 || dim > HNS_MAX_DIM || vdim < 1 ||
+      block_size < 1 || splits < 1 || kv_heads > 65535)
+    return TS_ERR_ARG;
+  if ((cos_table == nullptr) != (sin_table == nullptr) || (cos_table && (dim & 1))) return TS_ERR_ARG;
+  if ((q_gain == nullptr) != (k_gain == nullptr)) return TS_ERR_ARG;
+  if (slots && (!k_pages || !v_pages)) return TS_ERR_ARG;
+  if (dtype == TS_F32)
+    launch_head_norm_store<float, float>(q_out, q_stride, proj, splits, split_stride, k_pages, v_pages, q_gain, k_gain, eps, gain_offset, cos_table, sin_table, positions, slots, tokens, heads, kv_heads, dim, vdim, block_size, stream);
+  else if (dtype == TS_BF16 && in_f32)
+    launch_head_norm_store<bf16_t, float>(q_out, q_stride, proj, splits, split_stride, k_pages, v_pages, q_gain, k_gain, eps, gain_offset, cos_table, sin_table, positions, slots, tokens, heads, kv_heads, dim, vdim, block_size, stream);
+  else if (dtype == TS_BF16)
+    launch_head_norm_store<bf16_t, bf16_t>(q_out, q_stride, proj, splits, split_stride, k_pages, v_pages, q_gain, k_gain, eps, gain_offset, cos_table, sin_table, positions, slots, tokens, heads, kv_heads, dim, vdim, block_size, stream);
+  else
+    return TS_ERR_DTYPE;
+  return ts_launch_status();
+}

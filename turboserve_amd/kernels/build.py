@@ -33,6 +33,8 @@ ARCH = "gfx950"
 MODULES: dict[str, tuple[str, ...]] = {
     "core": (
         "elementwise.hip",
+        "head_norm_store.hip",
+        "moe.hip",
         "attention_generic.hip",
         "gemm_plain.hip",
         "gemm_skinny.hip",

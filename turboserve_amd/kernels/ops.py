@@ -40,17 +40,29 @@ def dtype_code(dtype: torch.dtype) -> int:
 _SIGNATURES: dict[str, dict[str, list]] = {
     "core": {
         "ts_embed": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
-        "ts_rmsnorm": [c_void_p, c_void_p, c_void_p, c_float, c_int, c_int, c_int, c_void_p],
+        "ts_rmsnorm": [c_void_p, c_void_p, c_void_p, c_float, c_int, c_int, c_float, c_int, c_int, c_void_p],
         "ts_add_rmsnorm": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_void_p, c_void_p, c_float,
-                           c_int, c_int, c_int, c_void_p],
-        "ts_swiglu": [c_void_p, c_void_p, c_int, c_int, c_long, c_int, c_int, c_int, c_int, c_void_p],
+                           c_int, c_int, c_float, c_int, c_int, c_void_p],
+        "ts_swiglu": [c_void_p, c_void_p, c_int, c_int, c_long, c_int, c_int, c_int, c_float, c_float, c_float, c_int,
+                      c_void_p],
         "ts_rope_store": [c_void_p, c_long, c_void_p, c_int, c_int, c_long, c_void_p, c_void_p, c_void_p, c_void_p,
                           c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
         "ts_gather_rows": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
         "ts_patch_tokens": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
         "ts_paged_attention_generic": [c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int,
-                                       c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
-                                       c_float, c_int, c_void_p, c_int, c_void_p],
+                                       c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
+                                       c_float, c_float, c_int, c_void_p, c_int, c_void_p],
+        "ts_head_norm_store": [c_void_p, c_long, c_void_p, c_int, c_int, c_long, c_void_p, c_void_p, c_void_p, c_void_p,
+                               c_float, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
+                               c_int, c_int, c_int, c_void_p],
+        "ts_embed_positions": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+        "ts_stream_offset": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+        "ts_moe_route": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
+                         c_int, c_float, c_int, c_void_p],
+        "ts_moe_pair_rows": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float,
+                             c_float, c_float, c_int, c_void_p],
+        "ts_moe_combine": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_void_p, c_int, c_int, c_int,
+                           c_int, c_void_p],
         "ts_gemm_plain": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_long, c_long,
                           c_int, c_int, c_void_p],
         "ts_gemm_tiled": [c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
@@ -129,12 +141,17 @@ def _i32(t: torch.Tensor | None, name: str) -> None:
         _need(t.dtype == torch.int32 and t.is_contiguous(), f"{name} must be contiguous int32")
 
 
-def _check_pages(k_pages: torch.Tensor, v_pages: torch.Tensor, dtype: torch.dtype) -> None:
-    """Key pages ``[NB, Hkv, BS, D]`` and transposed value pages ``[NB, Hkv, D, BS]``."""
+def _check_pages(k_pages: torch.Tensor, v_pages: torch.Tensor, dtype: torch.dtype, *, any_value_width: bool = False) -> None:
+    """Key pages ``[NB, Hkv, BS, D]`` and transposed value pages ``[NB, Hkv, D, BS]`` (with
+    ``any_value_width``: ``[NB, Hkv, Dv, BS]``)."""
     _need(k_pages.dim() == 4 and v_pages.dim() == 4 and k_pages.is_contiguous() and v_pages.is_contiguous()
           and k_pages.dtype == dtype and v_pages.dtype == dtype,
           "pages must be contiguous 4-d tensors of the queries' dtype")
     nb, kv_heads, block_size, head_dim = k_pages.shape
+    if any_value_width:
+        _need(v_pages.shape[0] == nb and v_pages.shape[1] == kv_heads and v_pages.shape[3] == block_size and v_pages.shape[2] >= 1,
+              "value pages must be [NB, Hkv, Dv, BS] for key pages [NB, Hkv, BS, D]")
+        return
     _need(tuple(v_pages.shape) == (nb, kv_heads, head_dim, block_size),
           "value pages must be [NB, Hkv, D, BS] for key pages [NB, Hkv, BS, D]")
 
@@ -315,14 +332,18 @@ class Ops:
                                   dtype_code(table.dtype), self.stream()), "ts_embed")
         return out
 
-    def rmsnorm(self, x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    def rmsnorm(self, x: torch.Tensor, weight: torch.Tensor, eps: float, *, gain_offset: float = 0.0,
+                one_rounding: bool = False) -> torch.Tensor:
+        """``weight * round(x * rsqrt(mean(x^2) + eps))`` or, with ``one_rounding``,
+        ``round(x * rsqrt(mean(x^2) + eps) * (gain_offset + weight))`` computed in 32-bit."""
         _gpu(x, weight)
         _need(x.dim() == 2 and x.is_contiguous(), "x must be contiguous [T, H]")
         _need(weight.shape == (x.shape[1],) and weight.dtype == x.dtype and weight.is_contiguous(),
               "weight must be [H] of x's dtype")
         y = torch.empty_like(x)
         _check(self.core.ts_rmsnorm(_ptr(y), _ptr(x), _ptr(weight), float(eps), x.shape[0], x.shape[1],
-                                    dtype_code(x.dtype), self.stream()), "ts_rmsnorm")
+                                    float(gain_offset), 1 if one_rounding else 0, dtype_code(x.dtype), self.stream()),
+               "ts_rmsnorm")
         return y
 
     @staticmethod
@@ -350,10 +371,14 @@ class Ops:
         weight: torch.Tensor,
         eps: float,
         rows: torch.Tensor | None = None,
+        *,
+        gain_offset: float = 0.0,
+        one_rounding: bool = False,
     ) -> torch.Tensor:
         """``residual += pending`` in 32-bit (in place) and the normalised sum in ``weight``'s
         dtype; with ``rows`` only those rows, and ``residual`` is left alone.  ``pending`` is a
-        ``[T, H]`` tensor of the run dtype or ``[S, T, H]`` 32-bit partial sums."""
+        ``[T, H]`` tensor of the run dtype or ``[S, T, H]`` 32-bit partial sums.  The gain is
+        applied as in :meth:`rmsnorm`."""
         _gpu(residual, pending, weight, rows)
         _i32(rows, "rows")
         _need(residual.dim() == 2 and residual.dtype == torch.float32 and residual.is_contiguous(),
@@ -366,15 +391,19 @@ class Ops:
         out_rows = tokens if rows is None else rows.numel()
         y = self.rows_buffer(out_rows, hidden, weight.dtype, residual.device)
         _check(self.core.ts_add_rmsnorm(_ptr(y), _ptr(residual), _ptr(pending), is_f32, splits, stride, _ptr(weight),
-                                        _ptr(rows), float(eps), out_rows, hidden, dtype_code(weight.dtype),
-                                        self.stream()), "ts_add_rmsnorm")
+                                        _ptr(rows), float(eps), out_rows, hidden, float(gain_offset),
+                                        1 if one_rounding else 0, dtype_code(weight.dtype), self.stream()),
+               "ts_add_rmsnorm")
         return y
 
-    def swiglu(self, gate_up: torch.Tensor, dtype: torch.dtype | None = None, *, paired: bool = False) -> torch.Tensor:
+    def swiglu(self, gate_up: torch.Tensor, dtype: torch.dtype | None = None, *, paired: bool = False,
+               rule: tuple[float, float, float] = (1.0, 0.0, 0.0)) -> torch.Tensor:
         """``silu(gate) * up`` of the fused ``[T, 2 I]`` projection (or its ``[S, T, 2 I]`` 32-bit
         partial sums) -> ``[T, I]`` of ``dtype`` (the projection's own if it is not partial).
         Gate fills the first ``I`` columns and up the last, or, with ``paired``, they alternate
-        (gate ``i`` in column ``2 i``, up ``i`` in column ``2 i + 1``)."""
+        (gate ``i`` in column ``2 i``, up ``i`` in column ``2 i + 1``).  ``rule = (steepness,
+        limit, up_shift)`` is the gated unit's: with ``g' = min(g, limit)`` and ``u' = clamp(u,
+        -limit, limit)`` where ``limit > 0``, ``g' * sigmoid(steepness * g') * (u' + up_shift)``."""
         _gpu(gate_up)
         tokens, width = gate_up.shape[-2], gate_up.shape[-1]
         _need(width % 2 == 0, "gate_up must be [T, 2 I]")
@@ -385,7 +414,8 @@ class Ops:
         inter = width // 2
         out = self.rows_buffer(tokens, inter, out_dtype, gate_up.device)
         _check(self.core.ts_swiglu(_ptr(out), _ptr(gate_up), is_f32, splits, stride, tokens, inter,
-                                   1 if paired else 0, dtype_code(out_dtype), self.stream()), "ts_swiglu")
+                                   1 if paired else 0, float(rule[0]), float(rule[1]), float(rule[2]),
+                                   dtype_code(out_dtype), self.stream()), "ts_swiglu")
         return out
 
     def gather_rows(self, x: torch.Tensor, rows: torch.Tensor) -> torch.Tensor:
@@ -464,6 +494,190 @@ class Ops:
                                        dtype_code(run_dtype), self.stream()), "ts_rope_store")
         return q_out, q_stride
 
+    def embed_positions(self, table: torch.Tensor, ids: torch.Tensor, positions: torch.Tensor,
+                        at: torch.Tensor) -> torch.Tensor:
+        """``float32 [T, H]``: row ``ids[t]`` of ``table [V, H]`` plus row ``positions[t]`` of the 32-bit
+        position table ``at [capacity, H]`` (the host keeps every position below its capacity)."""
+        _gpu(table, ids, positions, at)
+        _i32(ids, "ids")
+        _i32(positions, "positions")
+        _need(table.dim() == 2 and table.is_contiguous(), "table must be contiguous [V, H]")
+        tokens, (vocab, hidden) = ids.numel(), table.shape
+        _need(positions.numel() == tokens, "one position per token")
+        _need(at.dim() == 2 and at.shape[1] == hidden and at.dtype == torch.float32 and at.is_contiguous(),
+              "the position table must be contiguous float32 [capacity, H]")
+        out = torch.empty((tokens, hidden), dtype=torch.float32, device=table.device)
+        _check(self.core.ts_embed_positions(_ptr(out), _ptr(table), _ptr(ids), _ptr(positions), _ptr(at), tokens, hidden,
+                                            vocab, dtype_code(table.dtype), self.stream()), "ts_embed_positions")
+        return out
+
+    def stream_offset(self, residual: torch.Tensor, origin: torch.Tensor | None, offset: torch.Tensor | None) -> None:
+        """``residual [T, H] += origin [T, H] + offset [H]`` in 32-bit, in place (either addend may
+        be absent)."""
+        _gpu(residual, origin, offset)
+        _need(residual.dim() == 2 and residual.dtype == torch.float32 and residual.is_contiguous(),
+              "residual must be contiguous float32 [T, H]")
+        tokens, hidden = residual.shape
+        if origin is not None:
+            _need(origin.shape == residual.shape and origin.dtype == torch.float32 and origin.is_contiguous(),
+                  "origin must be float32 like the residual")
+        code = TS_F32
+        if offset is not None:
+            _need(offset.shape == (hidden,) and offset.is_contiguous(), "offset must be contiguous [H]")
+            code = dtype_code(offset.dtype)
+        _check(self.core.ts_stream_offset(_ptr(residual), _ptr(origin), _ptr(offset), tokens, hidden, code, self.stream()),
+               "ts_stream_offset")
+
+    def head_norm_store(
+        self,
+        proj: torch.Tensor,
+        k_pages: torch.Tensor | None,
+        v_pages: torch.Tensor | None,
+        q_gain: torch.Tensor | None,
+        k_gain: torch.Tensor | None,
+        eps: float,
+        positions: torch.Tensor,
+        slots: torch.Tensor | None,
+        heads: int,
+        kv_heads: int,
+        head_dim: int,
+        value_dim: int,
+        block_size: int,
+        dtype: torch.dtype | None = None,
+        *,
+        gain_offset: float = 0.0,
+        cos: torch.Tensor | None = None,
+        sin: torch.Tensor | None = None,
+        max_position: int = 0,
+    ) -> tuple[torch.Tensor, int]:
+        """Per-head norm of the q and k heads of the fused projection ``[T, Hq D + Hkv D + Hkv Dv]``
+        (``x * rsqrt(mean(x^2) + eps) * (gain_offset + gain)`` in 32-bit, the gain ``[D]`` shared by
+        the heads; no norm without gains), then the rotation by ``cos``/``sin [capacity, D/2]`` where
+        given, one rounding, and the store of k and v at ``slots`` into key pages ``[NB, Hkv, BS,
+        D]`` and value pages ``[NB, Hkv, Dv, BS]`` (skipped when ``slots`` is ``None``).  Returns
+        the tensor that holds the queries and its row stride, as :meth:`rope_store` does."""
+        _gpu(proj, k_pages, v_pages, q_gain, k_gain, positions, slots, cos, sin)
+        _i32(positions, "positions")
+        _i32(slots, "slots")
+        tokens = positions.numel()
+        width = (heads + kv_heads) * head_dim + kv_heads * value_dim
+        run_dtype = dtype or proj.dtype
+        if proj.dim() == 3:
+            _need(dtype is not None, "partial sums need the run dtype")
+        is_f32, splits, stride = self._partials(proj, tokens, width, run_dtype, "projection")
+        _need(1 <= head_dim <= ATTENTION_MAX_HEAD_DIM and value_dim >= 1, "head sizes outside what the kernel takes")
+        _need((q_gain is None) == (k_gain is None), "both gains or none")
+        for gain in (q_gain, k_gain):
+            if gain is not None:
+                _need(gain.shape == (head_dim,) and gain.dtype == run_dtype and gain.is_contiguous(),
+                      "a gain must be [D] of the run dtype")
+        if cos is not None:
+            _need(sin is not None and head_dim % 2 == 0 and cos.shape == sin.shape and cos.dim() == 2
+                  and cos.shape[1] == head_dim // 2 and cos.dtype == torch.float32 and sin.dtype == torch.float32
+                  and cos.is_contiguous() and sin.is_contiguous(), "cos/sin must be float32 [capacity, D/2]")
+            _need(max_position < cos.shape[0], f"position {max_position} is beyond the rotary tables ({cos.shape[0]})")
+        if slots is not None:
+            _need(slots.numel() == tokens, "one slot per token")
+            _need(k_pages is not None and v_pages is not None, "slots need pages")
+            _check_pages(k_pages, v_pages, run_dtype, any_value_width=True)
+            _need(k_pages.shape[1] == kv_heads and k_pages.shape[2] == block_size and k_pages.shape[3] == head_dim
+                  and v_pages.shape[2] == value_dim, "pages do not fit the heads")
+        if is_f32:
+            q_out = self.rows_buffer(tokens, heads * head_dim, run_dtype, proj.device)
+            q_stride = heads * head_dim
+        else:
+            q_out, q_stride = proj, width
+        _check(self.core.ts_head_norm_store(
+            _ptr(q_out), q_stride, _ptr(proj), is_f32, splits, stride, _ptr(k_pages), _ptr(v_pages), _ptr(q_gain),
+            _ptr(k_gain), float(eps), float(gain_offset), _ptr(cos), _ptr(sin), _ptr(positions), _ptr(slots), tokens,
+            heads, kv_heads, head_dim, value_dim, block_size, dtype_code(run_dtype), self.stream()), "ts_head_norm_store")
+        return q_out, q_stride
+
+    # -- routed feed-forward --------------------------------------------------------------------
+
+    def moe_route(self, x: torch.Tensor, router: torch.Tensor, *, top: int, groups: int, keep: int, scale: float,
+                  extra: torch.Tensor | None = None) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor | None]:
+        """The router of a routed feed-forward, in 32-bit: ``s = sigmoid(router x)``; the experts
+        form ``groups`` equal groups of neighbours, a group's mark is the sum of its two largest
+        ``s``, only the ``keep`` best groups' experts can be taken, the ``top`` of them with the
+        largest ``s`` are.  Returns ``(taken [T, top] int32, weights [T, top] float32, gate)``:
+        weights are ``s / (sum of the taken s + 1e-20) * scale``; ``gate [T]`` is
+        ``sigmoid(extra . x)`` for a vector ``extra [H]`` (``None`` without one)."""
+        _gpu(x, router, extra)
+        _need(x.dim() == 2 and x.is_contiguous() and router.dim() == 2 and router.is_contiguous()
+              and router.shape[1] == x.shape[1] and router.dtype == x.dtype, "x [T, H] and router [E, H] of one dtype")
+        tokens, hidden = x.shape
+        experts = router.shape[0]
+        _need(1 <= experts <= 1024 and 1 <= top <= 32 and groups >= 1 and experts % groups == 0 and 1 <= keep <= groups
+              and top <= (experts // groups) * keep, "a routing rule the kernel does not take")
+        taken = torch.empty((tokens, top), dtype=torch.int32, device=x.device)
+        weights = torch.empty((tokens, top), dtype=torch.float32, device=x.device)
+        gate = None
+        if extra is not None:
+            _need(extra.numel() == hidden and extra.dtype == x.dtype and extra.is_contiguous(), "extra must be [H]")
+            gate = torch.empty((tokens,), dtype=torch.float32, device=x.device)
+        _check(self.core.ts_moe_route(_ptr(taken), _ptr(weights), _ptr(gate), _ptr(x), _ptr(router), _ptr(extra), tokens,
+                                      hidden, experts, top, groups, keep, float(scale), dtype_code(x.dtype), self.stream()),
+               "ts_moe_route")
+        return taken, weights, gate
+
+    def moe_pair_rows(self, rows: torch.Tensor, weight: torch.Tensor, taken: torch.Tensor, *, share: int,
+                      rule: tuple[float, float, float] | None = None) -> torch.Tensor:
+        """The product of every (token, taken expert) pair with its expert's matrix out of the
+        stack ``weight [E, N, K]``: pair ``p`` (``taken.view(-1)[p]`` its expert) reads row ``p //
+        share`` of ``rows [*, K]``.  With ``rule`` the ``N = 2 I`` rows alternate gate, up and the
+        result is the gated unit, ``[P, I]`` of the run dtype; else ``[P, N]`` float32."""
+        _gpu(rows, weight, taken)
+        _i32(taken, "taken")
+        pairs = taken.numel()
+        _need(weight.dim() == 3 and weight.is_contiguous() and rows.dim() == 2 and rows.is_contiguous()
+              and rows.dtype == weight.dtype and rows.shape[1] == weight.shape[2], "rows [*, K] and weight [E, N, K] of one dtype")
+        experts, n, k = weight.shape
+        _need(share >= 1 and rows.shape[0] * share >= pairs and k <= 12288, "rows do not cover the pairs")
+        if rule is not None:
+            _need(n % 2 == 0, "a gated stack has an even number of rows")
+            out = torch.empty((pairs, n // 2), dtype=rows.dtype, device=rows.device)
+        else:
+            out = torch.empty((pairs, n), dtype=torch.float32, device=rows.device)
+        r = rule or (1.0, 0.0, 0.0)
+        _check(self.core.ts_moe_pair_rows(_ptr(out), _ptr(rows), _ptr(weight), _ptr(taken), pairs, share, n, k, experts,
+                                          0 if rule is None else 1, float(r[0]), float(r[1]), float(r[2]),
+                                          dtype_code(rows.dtype), self.stream()), "ts_moe_pair_rows")
+        return out
+
+    def moe_expert_units(self, x: torch.Tensor, gate_up: torch.Tensor, taken: torch.Tensor,
+                         rule: tuple[float, float, float]) -> torch.Tensor:
+        """The gated units ``[T * top, I]`` of every (token, taken expert) pair: ``x [T, H]`` against
+        the pair's expert's matrix of the stack ``gate_up [E, 2 I, H]`` (rows alternate gate, up)."""
+        return self.moe_pair_rows(x, gate_up, taken, share=taken.shape[1], rule=rule)
+
+    def moe_expert_outputs(self, units: torch.Tensor, down: torch.Tensor, taken: torch.Tensor) -> torch.Tensor:
+        """``[T * top, H]`` float32: every pair's units against its expert's matrix of ``down [E, H, I]``."""
+        return self.moe_pair_rows(units, down, taken, share=1)
+
+    def moe_combine(self, pair_out: torch.Tensor, weights: torch.Tensor, extra: torch.Tensor | None = None,
+                    extra_gate: torch.Tensor | None = None, dtype: torch.dtype | None = None) -> torch.Tensor:
+        """``[1, T, H]`` float32 (one partial sum for the residual stream): the pairs' outputs
+        ``[T * top, H]`` weighted by ``weights [T, top]`` and summed per token, plus ``extra_gate [T]``
+        times ``extra`` (``[T, H]`` of ``dtype`` or ``[S, T, H]`` 32-bit partial sums) where given."""
+        _gpu(pair_out, weights, extra, extra_gate)
+        tokens, top = weights.shape
+        _need(pair_out.dtype == torch.float32 and pair_out.is_contiguous() and pair_out.dim() == 2
+              and pair_out.shape[0] == tokens * top and weights.dtype == torch.float32 and weights.is_contiguous(),
+              "pair_out [T * top, H] and weights [T, top] must be float32")
+        hidden = pair_out.shape[1]
+        is_f32, splits, stride, code = 0, 1, 0, TS_F32
+        if extra is not None:
+            run = dtype or extra.dtype
+            is_f32, splits, stride = self._partials(extra, tokens, hidden, run, "extra")
+            code = dtype_code(run)
+        if extra_gate is not None:
+            _need(extra_gate.shape == (tokens,) and extra_gate.dtype == torch.float32, "extra_gate must be float32 [T]")
+        out = torch.empty((1, tokens, hidden), dtype=torch.float32, device=pair_out.device)
+        _check(self.core.ts_moe_combine(_ptr(out), _ptr(pair_out), _ptr(weights), _ptr(extra), is_f32, splits, stride,
+                                        _ptr(extra_gate), tokens, top, hidden, code, self.stream()), "ts_moe_combine")
+        return out
+
     # -- attention ----------------------------------------------------------------------------
 
     def paged_attention_generic(
@@ -479,8 +693,11 @@ class Ops:
         scale: float,
         window: int | None,
         slopes: torch.Tensor | None = None,
+        softcap: float = 0.0,
     ) -> torch.Tensor:
-        """Attention of every token over the keys ``lo..position`` of its request.
+        """Attention of every token over the keys ``lo..position`` of its request.  With
+        ``softcap = c > 0`` a scaled score ``s`` becomes ``c * tanh(s / c)``.  Values may have a
+        width of their own (value pages ``[NB, Hkv, Dv, BS]``); the result is ``[T, heads * Dv]``.
 
         ``q`` is the tensor whose first ``heads * D`` elements of each ``q_stride``-long row
         are the (already encoded) queries.  ``slopes [heads]`` (32-bit), if given, biases the
@@ -494,29 +711,32 @@ class Ops:
         _i32(block_table, "block_table")
         _i32(token_seq, "token_seq")
         _i32(positions, "positions")
-        _check_pages(k_pages, v_pages, q.dtype)
+        _check_pages(k_pages, v_pages, q.dtype, any_value_width=True)
         _, kv_heads, block_size, head_dim = k_pages.shape
+        value_dim = v_pages.shape[2]
+        _need(value_dim <= ATTENTION_MAX_HEAD_DIM, f"values of {value_dim} elements are wider than the kernel takes")
         tokens = positions.numel()
         _need(q.is_contiguous() and q.numel() >= tokens * q_stride and q_stride >= heads * head_dim,
               "q does not hold [T, q_stride] rows")
         _need(block_table.dim() == 2 and token_seq.numel() == tokens, "block_table [S, MB], token_seq [T]")
         _need(attention_geometry_error(heads, kv_heads, head_dim) is None,
               attention_geometry_error(heads, kv_heads, head_dim) or "")
-        out = self.rows_buffer(tokens, heads * head_dim, q.dtype, q.device)
+        out = self.rows_buffer(tokens, heads * value_dim, q.dtype, q.device)
         _check(self.core.ts_paged_attention_generic(
             _ptr(out), _ptr(q), q_stride, _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
-            block_table.shape[1], _ptr(token_seq), _ptr(positions), tokens, heads, kv_heads, head_dim,
-            block_size, float(scale), int(window or 0), _ptr(slopes) if slopes is not None else None,
+            block_table.shape[1], _ptr(token_seq), _ptr(positions), tokens, heads, kv_heads, head_dim, value_dim,
+            block_size, float(scale), float(softcap), int(window or 0), _ptr(slopes) if slopes is not None else None,
             dtype_code(q.dtype), self.stream()),
             "ts_paged_attention_generic")
         return out
 
     @staticmethod
-    def mfma_attention_supported(dtype: torch.dtype, head_dim: int, block_size: int) -> bool:
+    def mfma_attention_supported(dtype: torch.dtype, head_dim: int, block_size: int, softcap: float = 0.0) -> bool:
         """Whether the matrix-core attention kernels take this geometry (bfloat16, head sizes
-        16..256 in steps of 16, pages of at least 8 tokens); anything else runs the generic
-        kernel."""
-        return dtype == torch.bfloat16 and head_dim % 16 == 0 and 16 <= head_dim <= 256 and block_size >= 8
+        16..256 in steps of 16, pages of at least 8 tokens, no cap on the scores); anything else
+        runs the generic kernel."""
+        return (dtype == torch.bfloat16 and head_dim % 16 == 0 and 16 <= head_dim <= 256 and block_size >= 8
+                and not softcap)
 
     def attention_decode(
         self,
@@ -1150,11 +1370,15 @@ class Ops:
     #: 0.62% instead of 0.66%).
     library_residual_float32 = False
 
-    def linear_swiglu(self, x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+    def linear_swiglu(self, x: torch.Tensor, weight: torch.Tensor,
+                      rule: tuple[float, float, float] | None = None) -> torch.Tensor:
         """``silu(gate) * up`` of the projection of ``x`` by a gate|up matrix ``[2 I, K]`` whose rows
         alternate gate, up -> ``[T, I]`` in the dtype of ``x``.  Decode-sized bfloat16 batches whose
         product runs as one range of K get the activation in the product's own kernel; every other
-        case is the projection followed by :meth:`swiglu`."""
+        case is the projection followed by :meth:`swiglu`.  Another gated unit (``rule``, see
+        :meth:`swiglu`) is always the projection followed by the unit's kernel."""
+        if rule is not None and tuple(rule) != (1.0, 0.0, 0.0):
+            return self.swiglu(self.linear(x, weight), x.dtype, paired=True, rule=rule)
         if x.dtype == torch.bfloat16 and self.skinny_supported(x, weight) and x.shape[0] <= self.skinny_max_rows:
             _gpu(x, weight)
             if (self._few_rows_wide(x.shape[0], weight.shape[0], weight.shape[1], 1) and weight.shape[0] % 2 == 0

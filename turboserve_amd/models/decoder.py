@@ -25,6 +25,7 @@ from turboserve_amd.parts.base import (
     PartSpec,
     ResidualStream,
     Runtime,
+    StreamStep,
     TensorSpec,
 )
 from turboserve_amd.parts.registry import build_part
@@ -41,10 +42,14 @@ class LayerSpec:
 @dataclass(frozen=True)
 class LayerCall:
     """One entry of the run order: which layer runs and, optionally, the index of an EARLIER
-    entry whose cache it reads (it then writes nothing)."""
+    entry whose cache it reads (it then writes nothing).  ``enter``: a stream step (kind,
+    parameters and the checkpoint prefix of its tensors) that acts on the residual stream right
+    before this call: what a model adds when a pass through repeated layers begins."""
 
     layer: int
     cache_of: int | None = None
+    enter: PartSpec | None = None
+    enter_prefix: str = ""
 
 
 @dataclass(frozen=True)
@@ -81,6 +86,12 @@ class DecoderModel:
         ]
         self.embedding: Embedding = build_part("embedding", plan.embedding, plan.embedding_prefix, runtime)
         self.head: Head = build_part("head", plan.head, plan.head_prefix, runtime)
+        #: per schedule entry: the stream step that runs before it, or None
+        self.enter_steps: list[StreamStep | None] = [
+            None if call.enter is None else build_part("stream_step", call.enter, call.enter_prefix, runtime)
+            for call in plan.schedule
+        ]
+        self.keeps_origin = any(step is not None and step.needs_origin for step in self.enter_steps)
 
     # -- weights ------------------------------------------------------------------------------
 
@@ -89,6 +100,12 @@ class DecoderModel:
         specs: dict[str, TensorSpec] = dict(self.embedding.tensor_specs())
         for block in self.blocks:
             specs.update(block.tensor_specs())
+        for step in self.enter_steps:
+            for name, spec in (step.tensor_specs() if step is not None else {}).items():
+                # Steps may share a tensor (the passes of one loop: rows of one table).
+                if name in specs and specs[name] != spec:
+                    raise ValueError(f"a stream step expects {spec} under {name!r}, another part {specs[name]}")
+                specs[name] = spec
         for name, spec in self.head.tensor_specs().items():
             # A head may name a tensor of another part (a tied head: the token table) and then
             # shares it; both must expect the same thing there.
@@ -106,6 +123,9 @@ class DecoderModel:
         self.embedding.load(tensors)
         for block in self.blocks:
             block.load(tensors)
+        for step in self.enter_steps:
+            if step is not None:
+                step.load(tensors)
         self.head.load(tensors)
 
     def num_parameters(self) -> int:
@@ -125,7 +145,7 @@ class DecoderModel:
         working copy (the reference's estimate has the same terms from Qwen2's sizes,
         src/turboserve/engine/runtime/memory.py:208-242)."""
         plan = self.plan
-        stream = tokens * plan.hidden_size * (4 + 4)
+        stream = tokens * plan.hidden_size * (4 + 4 + (4 if self.keeps_origin else 0))
         layer = max((block.activation_bytes(tokens, itemsize) for block in self.blocks), default=0)
         layer += self.head.activation_bytes(tokens, itemsize)
         return 2 * (stream + layer) + requests * plan.vocab_size * 4 * 2
@@ -136,7 +156,7 @@ class DecoderModel:
         """Whether single-token steps of this model may be recorded into HIP graphs: every
         part says so (``Part.capturable``)."""
         return (all(block.is_capturable() for block in self.blocks) and self.embedding.is_capturable()
-                and self.head.is_capturable())
+                and self.head.is_capturable() and all(step is None or step.is_capturable() for step in self.enter_steps))
 
     def step_fields(self) -> tuple:
         """The integer fields the model's parts want in every step's packed buffer beside the
@@ -146,6 +166,9 @@ class DecoderModel:
         asked = [*self.embedding.step_fields()]
         for block in self.blocks:
             asked.extend(block.step_fields())
+        for step in self.enter_steps:
+            if step is not None:
+                asked.extend(step.step_fields())
         asked.extend(self.head.step_fields())
         return merge_step_fields(asked)
 
@@ -165,7 +188,11 @@ class DecoderModel:
         if len(caches) != len(self.plan.schedule):
             raise ValueError(f"{len(caches)} cache views for {len(self.plan.schedule)} scheduled layer calls")
         stream = ResidualStream(self.embedding.forward(token_ids, ctx))
-        for call, cache in zip(self.plan.schedule, caches):
+        # The embedding's output is kept apart only where a stream step adds it in again later.
+        origin = stream.residual.clone() if self.keeps_origin else None
+        for call, cache, enter in zip(self.plan.schedule, caches, self.enter_steps):
+            if enter is not None:
+                stream = enter.forward(stream, ctx, origin)
             stream = self.blocks[call.layer].forward(stream, ctx, cache)
         return stream
 

@@ -1,6 +1,6 @@
 """The parts a model is assembled from; importing this package registers the built-in kinds."""
 
-from turboserve_amd.parts import attention, block, ends, mlp, norm, rope  # noqa: F401  (registration)
+from turboserve_amd.parts import attention, block, ends, experts, mlp, norm, rope, stream  # noqa: F401  (registration)
 from turboserve_amd.parts.base import (  # noqa: F401
     Block,
     CacheNeed,
@@ -18,6 +18,7 @@ from turboserve_amd.parts.base import (  # noqa: F401
     PositionEncoding,
     ResidualStream,
     Runtime,
+    StreamStep,
     TensorSpec,
 )
 from turboserve_amd.parts.registry import (  # noqa: F401
@@ -29,4 +30,5 @@ from turboserve_amd.parts.registry import (  # noqa: F401
     register_mixer,
     register_norm,
     register_position_encoding,
+    register_stream_step,
 )

@@ -20,7 +20,16 @@ class GroupedQueryAttention(Mixer):
 
     The three projections are held as one ``[(Hq + 2 Hkv) D, H]`` matrix (the checkpoint keeps
     them apart; ``load`` concatenates), so a step does one product for them.  Scale is a
-    parameter (``head_dim ** -0.5`` for Qwen2, model_config.py:224-227)."""
+    parameter (``head_dim ** -0.5`` for Qwen2, model_config.py:224-227).
+
+    Optional, each a parameter of its own: ``value_dim`` (values of another width than the keys:
+    the fused matrix is ``[Hq D + Hkv D + Hkv Dv, H]`` and the output projection reads ``Hq Dv``);
+    ``head_norm = {"eps": e, "gain_offset": o}`` (every q and k head is divided by its root mean
+    square, eps inside the root, and multiplied by ``o +`` a gain vector ``[D]`` that all heads
+    share, one for q and one for k, in 32-bit, before the position encoding); ``softcap = c``
+    (a scaled score ``s`` becomes ``c * tanh(s / c)`` before the softmax).  ``names``: the tensor
+    names under the part's prefix of ``q, k, v, o`` (biases: the same with ``weight`` replaced by
+    ``bias``) and of the two gains."""
 
     def __init__(
         self,
@@ -36,6 +45,10 @@ class GroupedQueryAttention(Mixer):
         out_bias: bool,
         window: int | None,
         position: PartSpec,
+        value_dim: int | None = None,
+        head_norm: Mapping | None = None,
+        softcap: float = 0.0,
+        names: Mapping[str, str] | None = None,
     ) -> None:
         super().__init__(prefix, runtime)
         # Refused here, when the model is put together, not at the first step after the weights
@@ -52,15 +65,28 @@ class GroupedQueryAttention(Mixer):
         self.out_bias = bool(out_bias)
         self.window = None if window is None else int(window)
         self.position = build_part("position_encoding", position, prefix, runtime)
+        self.value_dim = self.head_dim if value_dim is None else int(value_dim)
+        if not 1 <= self.value_dim <= 512:
+            raise ValueError(f"{prefix or 'attention'}: values of {self.value_dim} elements are outside what the kernels take")
+        self.softcap = float(softcap)
+        self.head_norm_eps = None if head_norm is None else float(head_norm["eps"])
+        self.head_norm_offset = 0.0 if head_norm is None else float(head_norm.get("gain_offset", 0.0))
+        self.names = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight",
+                      "q_norm": "q_norm.weight", "k_norm": "k_norm.weight", **(names or {})}
         self.q_size = self.num_heads * self.head_dim
         self.kv_size = self.num_kv_heads * self.head_dim
+        self.v_size = self.num_kv_heads * self.value_dim
+        self.out_size = self.num_heads * self.value_dim
+        self.q_gain: torch.Tensor | None = None
+        self.k_gain: torch.Tensor | None = None
         self.qkv_weight: torch.Tensor | None = None
         self.qkv_bias_tensor: torch.Tensor | None = None
         self.o_weight: torch.Tensor | None = None
         self.o_bias_tensor: torch.Tensor | None = None
 
     def cache_need(self) -> CacheNeed:
-        return PagedKV(self.num_kv_heads, self.head_dim, self.window)
+        return PagedKV(self.num_kv_heads, self.head_dim, self.window,
+                       None if self.value_dim == self.head_dim else self.value_dim)
 
     def is_capturable(self) -> bool:
         return self.capturable and self.position.is_capturable()
@@ -71,42 +97,60 @@ class GroupedQueryAttention(Mixer):
     def activation_bytes(self, tokens: int, itemsize: int) -> int:
         """The fused projection, the attention output and the output projection (32-bit: it is
         added to the residual stream) of a step."""
-        return tokens * ((self.q_size + 2 * self.kv_size + self.q_size) * itemsize + self.hidden_size * 4)
+        return tokens * ((self.q_size + self.kv_size + self.v_size + self.out_size) * itemsize + self.hidden_size * 4)
 
     def tensor_specs(self) -> dict[str, TensorSpec]:
         specs = {
-            self.name("q_proj.weight"): TensorSpec((self.q_size, self.hidden_size)),
-            self.name("k_proj.weight"): TensorSpec((self.kv_size, self.hidden_size)),
-            self.name("v_proj.weight"): TensorSpec((self.kv_size, self.hidden_size)),
-            self.name("o_proj.weight"): TensorSpec((self.hidden_size, self.q_size)),
+            self.name(self.names["q"]): TensorSpec((self.q_size, self.hidden_size)),
+            self.name(self.names["k"]): TensorSpec((self.kv_size, self.hidden_size)),
+            self.name(self.names["v"]): TensorSpec((self.v_size, self.hidden_size)),
+            self.name(self.names["o"]): TensorSpec((self.hidden_size, self.out_size)),
         }
         if self.qkv_bias:
-            specs[self.name("q_proj.bias")] = TensorSpec((self.q_size,))
-            specs[self.name("k_proj.bias")] = TensorSpec((self.kv_size,))
-            specs[self.name("v_proj.bias")] = TensorSpec((self.kv_size,))
+            specs[self.name(self._bias("q"))] = TensorSpec((self.q_size,))
+            specs[self.name(self._bias("k"))] = TensorSpec((self.kv_size,))
+            specs[self.name(self._bias("v"))] = TensorSpec((self.v_size,))
         if self.out_bias:
-            specs[self.name("o_proj.bias")] = TensorSpec((self.hidden_size,))
+            specs[self.name(self._bias("o"))] = TensorSpec((self.hidden_size,))
+        if self.head_norm_eps is not None:
+            init = "zeros" if self.head_norm_offset == 1.0 else "ones"
+            specs[self.name(self.names["q_norm"])] = TensorSpec((self.head_dim,), init=init)
+            specs[self.name(self.names["k_norm"])] = TensorSpec((self.head_dim,), init=init)
         specs.update(self.position.tensor_specs())
         return specs
 
+    def _bias(self, which: str) -> str:
+        name = self.names[which]
+        if "weight" not in name:
+            raise ValueError(f"{self.prefix}: no bias name can be made from the tensor name {name!r}")
+        return name.replace("weight", "bias")
+
     def load(self, tensors: Mapping[str, torch.Tensor]) -> None:
         self.qkv_weight = torch.cat(
-            [tensors[self.name(f"{p}_proj.weight")] for p in ("q", "k", "v")], dim=0
+            [tensors[self.name(self.names[p])] for p in ("q", "k", "v")], dim=0
         ).contiguous()
         if self.qkv_bias:
             self.qkv_bias_tensor = torch.cat(
-                [tensors[self.name(f"{p}_proj.bias")] for p in ("q", "k", "v")], dim=0
+                [tensors[self.name(self._bias(p))] for p in ("q", "k", "v")], dim=0
             ).contiguous()
-        self.o_weight = tensors[self.name("o_proj.weight")].contiguous()
+        self.o_weight = tensors[self.name(self.names["o"])].contiguous()
         if self.out_bias:
-            self.o_bias_tensor = tensors[self.name("o_proj.bias")].contiguous()
+            self.o_bias_tensor = tensors[self.name(self._bias("o"))].contiguous()
+        if self.head_norm_eps is not None:
+            self.q_gain = tensors[self.name(self.names["q_norm"])].contiguous()
+            self.k_gain = tensors[self.name(self.names["k_norm"])].contiguous()
         self.position.load(tensors)
 
     def forward(self, x: torch.Tensor, ctx, cache: PagedKVView) -> torch.Tensor:
         ops = self.runtime.ops
         qkv = ops.linear(x, self.qkv_weight, self.qkv_bias_tensor)
+        more = {}
+        if self.value_dim != self.head_dim:
+            more["value_dim"] = self.value_dim
+        if self.head_norm_eps is not None:
+            more["head_norm"] = (self.q_gain, self.k_gain, self.head_norm_eps, self.head_norm_offset)
         q, q_stride = self.position.encode_and_store(
-            qkv, self.num_heads, self.num_kv_heads, self.head_dim, ctx, cache
+            qkv, self.num_heads, self.num_kv_heads, self.head_dim, ctx, cache, **more
         )
         attended = self.attend(q, q_stride, ctx, cache)
         return ops.linear(attended, self.o_weight, self.o_bias_tensor, for_residual=True)
@@ -122,7 +166,8 @@ class GroupedQueryAttention(Mixer):
         ops = self.runtime.ops
         table = ctx.block_tables[cache.group]
         slopes = self.position.score_slopes(self.num_heads)
-        fast = slopes is None and ops.mfma_attention_supported(qkv.dtype, self.head_dim, cache.block_size)
+        fast = (slopes is None and self.value_dim == self.head_dim
+                and ops.mfma_attention_supported(qkv.dtype, self.head_dim, cache.block_size, self.softcap))
         if fast:
             out = ops.rows_buffer(ctx.num_tokens, self.q_size, qkv.dtype, qkv.device)
             if ctx.num_prefill_seqs > 0:
@@ -146,5 +191,5 @@ class GroupedQueryAttention(Mixer):
             return out
         return ops.paged_attention_generic(
             qkv, q_stride, cache.k, cache.v, table, ctx.token_seq, ctx.positions,
-            self.num_heads, self.scale, self.window, slopes,
+            self.num_heads, self.scale, self.window, slopes, self.softcap,
         )

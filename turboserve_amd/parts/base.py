@@ -157,6 +157,10 @@ class Part:
         self.runtime = runtime
 
     def name(self, suffix: str) -> str:
+        """The checkpoint name of a tensor of this part; an empty suffix names the prefix itself (a
+        part whose one tensor is stored under the part's own name)."""
+        if not suffix:
+            return self.prefix
         return f"{self.prefix}.{suffix}" if self.prefix else suffix
 
     def is_capturable(self) -> bool:
@@ -210,11 +214,18 @@ class PositionEncoding(Part):
         head_dim: int,
         ctx: "StepContext",
         cache: PagedKVView,
+        **more: Any,
     ) -> tuple[torch.Tensor, int]:
         """``qkv``: the fused projection ``[T, (Hq + 2 Hkv) D]`` as ``ops.linear`` returned it (a
         tensor of the run dtype, or 32-bit partial sums ``[S, T, ..]``).  Encodes q and k, writes
         k, v at the step's slots of ``cache.group`` unless the cache is not writable, and
-        returns the tensor holding the encoded queries with its row stride."""
+        returns the tensor holding the encoded queries with its row stride.
+
+        A mixer that needs more of the same pass says so in ``more`` (and only then, so an
+        encoding that knows nothing of these is still usable by the mixers that do not):
+        ``value_dim`` (values ``Dv`` wide, the projection being ``[T, Hq D + Hkv D + Hkv Dv]``) and
+        ``head_norm = (q_gain [D], k_gain [D], eps, gain_offset)`` (every q and k head is divided
+        by its root mean square and multiplied by ``gain_offset + gain`` before the encoding)."""
         raise NotImplementedError
 
     def score_slopes(self, num_heads: int) -> torch.Tensor | None:
@@ -260,6 +271,19 @@ class Mixer(Part):
         ``ops.linear``, ``[S, T, H]`` 32-bit partial sums).  The rows of request ``s`` are
         ``ctx.query_start_loc[s]:ctx.query_start_loc[s+1]``, in position order, continuing
         whatever earlier steps left in ``cache``."""
+        raise NotImplementedError
+
+
+class StreamStep(Part):
+    """Acts on the residual stream between two layer calls (an offset added when a pass through
+    repeated layers begins, a re-injection of the embedding)."""
+
+    #: Whether ``forward`` wants the embedding's output of this step (the model then keeps it).
+    needs_origin = False
+
+    def forward(self, stream: ResidualStream, ctx: "StepContext", origin: torch.Tensor | None) -> ResidualStream:
+        """``origin``: the 32-bit ``[T, H]`` the embedding made for this step, or ``None`` when no
+        step of the plan asked for it."""
         raise NotImplementedError
 
 

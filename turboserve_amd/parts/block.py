@@ -17,7 +17,8 @@ class PreNormBlock(Block):
     The sums are carried in the 32-bit residual stream; each part's output waits in
     ``stream.pending`` until the next norm adds it, in the same pass that normalises.
     ``mixer_norm_name`` / ``ff_norm_name`` / ``mixer_name`` / ``ff_name`` are the checkpoint
-    names of the four parts under the block's prefix."""
+    names of the four parts under the block's prefix.  A block without a feed-forward
+    (``feed_forward=None``) is its first half alone and has no second norm."""
 
     def __init__(
         self,
@@ -25,9 +26,9 @@ class PreNormBlock(Block):
         runtime: Runtime,
         *,
         mixer: PartSpec,
-        feed_forward: PartSpec,
+        feed_forward: PartSpec | None,
         mixer_norm: PartSpec,
-        ff_norm: PartSpec,
+        ff_norm: PartSpec | None,
         mixer_name: str = "self_attn",
         ff_name: str = "mlp",
         mixer_norm_name: str = "input_layernorm",
@@ -36,18 +37,24 @@ class PreNormBlock(Block):
         super().__init__(prefix, runtime)
         self.mixer_norm = build_part("norm", mixer_norm, self.name(mixer_norm_name), runtime)
         self.mixer = build_part("mixer", mixer, self.name(mixer_name), runtime)
-        self.ff_norm = build_part("norm", ff_norm, self.name(ff_norm_name), runtime)
-        self.feed_forward = build_part("feed_forward", feed_forward, self.name(ff_name), runtime)
+        self.ff_norm = self.feed_forward = None
+        if feed_forward is not None:
+            if ff_norm is None:
+                raise ValueError(f"{prefix}: a feed-forward needs its norm")
+            self.ff_norm = build_part("norm", ff_norm, self.name(ff_norm_name), runtime)
+            self.feed_forward = build_part("feed_forward", feed_forward, self.name(ff_name), runtime)
 
     def parts(self) -> list[Part]:
+        if self.feed_forward is None:
+            return [self.mixer_norm, self.mixer]
         return [self.mixer_norm, self.mixer, self.ff_norm, self.feed_forward]
 
     def activation_bytes(self, tokens: int, itemsize: int) -> int:
         """A norm's output stays alive while the part it feeds runs."""
-        return max(
-            self.mixer_norm.activation_bytes(tokens, itemsize) + self.mixer.activation_bytes(tokens, itemsize),
-            self.ff_norm.activation_bytes(tokens, itemsize) + self.feed_forward.activation_bytes(tokens, itemsize),
-        )
+        first = self.mixer_norm.activation_bytes(tokens, itemsize) + self.mixer.activation_bytes(tokens, itemsize)
+        if self.feed_forward is None:
+            return first
+        return max(first, self.ff_norm.activation_bytes(tokens, itemsize) + self.feed_forward.activation_bytes(tokens, itemsize))
 
     def tensor_specs(self) -> dict[str, TensorSpec]:
         specs: dict[str, TensorSpec] = {}
@@ -62,6 +69,8 @@ class PreNormBlock(Block):
     def forward(self, stream: ResidualStream, ctx, cache: CacheView) -> ResidualStream:
         x = self.mixer_norm.forward_residual(stream)
         stream.pending = self.mixer.forward(x, ctx, cache)
+        if self.feed_forward is None:
+            return stream
         x = self.ff_norm.forward_residual(stream)
         stream.pending = self.feed_forward.forward(x, ctx)
         return stream

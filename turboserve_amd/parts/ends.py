@@ -14,22 +14,67 @@ from turboserve_amd.parts.registry import build_part, register_embedding, regist
 
 @register_embedding("token_table")
 class TokenTable(Embedding):
-    """One row of ``[V, H]`` per token id, into the 32-bit residual stream."""
+    """One row of ``[V, H]`` per token id, into the 32-bit residual stream.  ``weight_name``: the
+    table's name under the part's prefix (empty: the prefix itself)."""
 
-    def __init__(self, prefix: str, runtime: Runtime, *, vocab_size: int, hidden_size: int) -> None:
+    def __init__(self, prefix: str, runtime: Runtime, *, vocab_size: int, hidden_size: int,
+                 weight_name: str = "weight") -> None:
         super().__init__(prefix, runtime)
         self.vocab_size = int(vocab_size)
         self.hidden_size = int(hidden_size)
+        self.weight_name = weight_name
         self.weight: torch.Tensor | None = None
 
     def tensor_specs(self) -> dict[str, TensorSpec]:
-        return {self.name("weight"): TensorSpec((self.vocab_size, self.hidden_size))}
+        return {self.name(self.weight_name): TensorSpec((self.vocab_size, self.hidden_size))}
 
     def load(self, tensors: Mapping[str, torch.Tensor]) -> None:
-        self.weight = tensors[self.name("weight")].contiguous()
+        self.weight = tensors[self.name(self.weight_name)].contiguous()
 
     def forward(self, token_ids: torch.Tensor, ctx) -> torch.Tensor:
         return self.runtime.ops.embed(self.weight, token_ids)
+
+
+def sinusoid_table(capacity: int, width: int, base: float) -> torch.Tensor:
+    """32-bit ``[capacity, width]``: entry ``2i`` of row ``p`` is ``sin(p * base^(-2i/width))``, entry
+    ``2i + 1`` the cosine of the same angle.  Angles are formed in 64-bit on the CPU and the
+    results rounded once, so a row does not depend on how far the table reaches."""
+    pairs = (width + 1) // 2
+    rates = torch.tensor(base, dtype=torch.float64) ** (-2.0 * torch.arange(pairs, dtype=torch.float64) / width)
+    angles = torch.outer(torch.arange(capacity, dtype=torch.float64), rates)
+    table = torch.stack([angles.sin(), angles.cos()], dim=2).reshape(capacity, 2 * pairs)[:, :width]
+    return table.to(torch.float32).contiguous()
+
+
+@register_embedding("token_table_sinusoid")
+class SinusoidTokenTable(TokenTable):
+    """A token's row of the table plus the sinusoidal vector of its position
+    (:func:`sinusoid_table`), summed in 32-bit.  The position table is made at the first step for
+    ``max_positions`` rows and grows by doubling when a step reaches further; a recorded step
+    holds the address of the table it was recorded with, so superseded tables are kept (they
+    cover every position such a recording can bring)."""
+
+    def __init__(self, prefix: str, runtime: Runtime, *, vocab_size: int, hidden_size: int, base: float = 10000.0,
+                 max_positions: int = 4096, weight_name: str = "weight") -> None:
+        super().__init__(prefix, runtime, vocab_size=vocab_size, hidden_size=hidden_size, weight_name=weight_name)
+        self.base = float(base)
+        self.initial_capacity = int(max_positions)
+        self.capacity = 0
+        self.at: torch.Tensor | None = None
+        self.superseded: list[torch.Tensor] = []
+
+    def ensure_capacity(self, num_positions: int) -> None:
+        if num_positions <= self.capacity:
+            return
+        target = max(num_positions, 2 * self.capacity, self.initial_capacity, 16)
+        if self.at is not None:
+            self.superseded.append(self.at)
+        self.at = sinusoid_table(target, self.hidden_size, self.base).to(self.runtime.device)
+        self.capacity = target
+
+    def forward(self, token_ids: torch.Tensor, ctx) -> torch.Tensor:
+        self.ensure_capacity(ctx.max_context_len)
+        return self.runtime.ops.embed_positions(self.weight, token_ids, ctx.positions, self.at)
 
 
 @register_head("norm_linear")
@@ -49,8 +94,10 @@ class NormLinearHead(Head):
         norm: PartSpec,
         norm_prefix: str,
         tied_to: str | None,
+        weight_name: str = "weight",
     ) -> None:
         super().__init__(prefix, runtime)
+        self.own_weight_name = weight_name
         self.vocab_size = int(vocab_size)
         self.hidden_size = int(hidden_size)
         self.norm = build_part("norm", norm, norm_prefix, runtime)
@@ -59,7 +106,7 @@ class NormLinearHead(Head):
 
     @property
     def weight_name(self) -> str:
-        return self.tied_to or self.name("weight")
+        return self.tied_to or self.name(self.own_weight_name)
 
     def is_capturable(self) -> bool:
         return self.capturable and self.norm.is_capturable()
@@ -70,7 +117,7 @@ class NormLinearHead(Head):
         return specs
 
     def ignorable_names(self) -> set[str]:
-        return {self.name("weight")} if self.tied_to else set()
+        return {self.name(self.own_weight_name)} if self.tied_to else set()
 
     def load(self, tensors: Mapping[str, torch.Tensor]) -> None:
         self.norm.load(tensors)

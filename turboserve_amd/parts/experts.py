@@ -1,0 +1,125 @@
+"""A routed feed-forward: many small gated feed-forwards ("experts"), of which each token takes a
+few, chosen by a router; optionally one more that every token takes."""
+
+from __future__ import annotations
+
+from collections.abc import Mapping
+
+import torch
+
+from turboserve_amd.parts.base import FeedForward, PartSpec, Runtime, TensorSpec
+from turboserve_amd.parts.registry import build_part, register_feed_forward
+
+
+@register_feed_forward("routed_experts")
+class RoutedExperts(FeedForward):
+    """``sum_j w_j * expert_{e_j}(x)  (+ gate(x) * shared(x))``.
+
+    Router, in 32-bit: ``s = sigmoid(router x)``.  The ``experts`` form ``groups`` equal groups
+    of neighbours; a group's mark is the sum of its two largest ``s``; only experts of the
+    ``keep`` groups with the largest marks can be taken; the ``top`` of them with the largest
+    ``s`` are, with weights ``s / (sum of the taken s + 1e-20) * route_scale`` (``groups = keep
+    = 1`` is plain top-k).  An expert is ``down(g * sigmoid(steepness g) * (u + up_shift))`` by
+    ``rule`` as in the ``swiglu`` part.  ``shared``: the ``PartSpec`` of a feed-forward every
+    token runs through, under ``<prefix>.<shared_name>``; with ``shared_gate_name`` its output
+    is multiplied by ``sigmoid(v . x)``, one number per token, ``v`` the tensor of that name.
+
+    The experts' matrices are stacked at load: ``[E, 2 I, H]`` with rows alternating gate, up,
+    and ``[E, H, I]``.  A step routes on the device, runs every (token, taken expert) pair
+    against its expert's matrices and sums with the weights, so nothing depends on data the
+    host has not seen and single-token steps can be recorded.
+    """
+
+    def __init__(
+        self,
+        prefix: str,
+        runtime: Runtime,
+        *,
+        hidden_size: int,
+        expert_size: int,
+        experts: int,
+        top: int,
+        groups: int = 1,
+        keep: int = 1,
+        route_scale: float = 1.0,
+        rule: tuple[float, float, float] = (1.0, 0.0, 0.0),
+        shared: PartSpec | None = None,
+        shared_name: str = "shared",
+        shared_gate_name: str | None = None,
+        router_name: str = "router",
+        expert_names: tuple[str, str, str, str] = ("e{index}", "gate", "up", "down"),
+    ) -> None:
+        super().__init__(prefix, runtime)
+        self.hidden_size = int(hidden_size)
+        self.expert_size = int(expert_size)
+        self.experts = int(experts)
+        self.top = int(top)
+        self.groups = int(groups)
+        self.keep = int(keep)
+        self.route_scale = float(route_scale)
+        self.rule = tuple(float(v) for v in rule)
+        if self.experts < 1 or self.groups < 1 or self.experts % self.groups != 0:
+            raise ValueError(f"{prefix}: {self.experts} experts do not form {self.groups} equal groups")
+        if not 1 <= self.keep <= self.groups:
+            raise ValueError(f"{prefix}: {self.keep} of {self.groups} groups cannot be kept")
+        if not 1 <= self.top <= (self.experts // self.groups) * self.keep:
+            raise ValueError(f"{prefix}: {self.top} experts cannot be taken from {self.keep} groups of {self.experts // self.groups}")
+        if self.experts > 1024 or self.top > 32:
+            raise ValueError(f"{prefix}: the router's kernel takes up to 1,024 experts and 32 per token")
+        self.router_name = router_name
+        self.expert_names = tuple(expert_names)
+        self.shared = None if shared is None else build_part("feed_forward", shared, self.name(shared_name), runtime)
+        self.shared_gate_name = None if shared is None or not shared_gate_name else self.shared.name(shared_gate_name)
+        self.router: torch.Tensor | None = None
+        self.shared_gate: torch.Tensor | None = None
+        self.gate_up: torch.Tensor | None = None   # [E, 2 I, H], rows alternate gate, up
+        self.down: torch.Tensor | None = None      # [E, H, I]
+
+    def _expert(self, index: int, which: int) -> str:
+        return self.name(f"{self.expert_names[0].format(index=index)}.{self.expert_names[which]}")
+
+    def is_capturable(self) -> bool:
+        return self.capturable and (self.shared is None or self.shared.is_capturable())
+
+    def tensor_specs(self) -> dict[str, TensorSpec]:
+        specs = {self.name(self.router_name): TensorSpec((self.experts, self.hidden_size))}
+        for index in range(self.experts):
+            specs[self._expert(index, 1)] = TensorSpec((self.expert_size, self.hidden_size))
+            specs[self._expert(index, 2)] = TensorSpec((self.expert_size, self.hidden_size))
+            specs[self._expert(index, 3)] = TensorSpec((self.hidden_size, self.expert_size))
+        if self.shared is not None:
+            specs.update(self.shared.tensor_specs())
+        if self.shared_gate_name:
+            specs[self.shared_gate_name] = TensorSpec((1, self.hidden_size))
+        return specs
+
+    def activation_bytes(self, tokens: int, itemsize: int) -> int:
+        """Per pair the gated units and the 32-bit output; per token the 32-bit sum; the shared
+        feed-forward runs while the pairs' outputs are held."""
+        pairs = tokens * self.top
+        own = pairs * (self.expert_size * itemsize + self.hidden_size * 4) + tokens * self.hidden_size * 4
+        return own + (self.shared.activation_bytes(tokens, itemsize) if self.shared is not None else 0)
+
+    def load(self, tensors: Mapping[str, torch.Tensor]) -> None:
+        self.router = tensors[self.name(self.router_name)].contiguous()
+        first = tensors[self._expert(0, 1)]
+        self.gate_up = torch.empty((self.experts, 2 * self.expert_size, self.hidden_size), dtype=first.dtype, device=first.device)
+        self.down = torch.empty((self.experts, self.hidden_size, self.expert_size), dtype=first.dtype, device=first.device)
+        for index in range(self.experts):
+            self.gate_up[index, 0::2] = first if index == 0 else tensors[self._expert(index, 1)]
+            self.gate_up[index, 1::2] = tensors[self._expert(index, 2)]
+            self.down[index] = tensors[self._expert(index, 3)]
+        del first
+        if self.shared is not None:
+            self.shared.load(tensors)
+        if self.shared_gate_name:
+            self.shared_gate = tensors[self.shared_gate_name].reshape(-1).contiguous()
+
+    def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
+        ops = self.runtime.ops
+        taken, weights, gate = ops.moe_route(x, self.router, top=self.top, groups=self.groups, keep=self.keep,
+                                             scale=self.route_scale, extra=self.shared_gate)
+        units = ops.moe_expert_units(x, self.gate_up, taken, self.rule)
+        outputs = ops.moe_expert_outputs(units, self.down, taken)
+        extra = self.shared.forward(x, ctx) if self.shared is not None else None
+        return ops.moe_combine(outputs, weights, extra, gate, x.dtype)

@@ -15,20 +15,29 @@ class SwiGLU(FeedForward):
     """``down(silu(gate(x)) * up(x))`` (layers.py:437-440).  Gate and up are held as one
     ``[2 I, H]`` matrix whose rows alternate gate, up (interleaved at load; the checkpoint keeps
     them apart): a step does one product for both, and the product's kernel has each gate
-    value next to its up value, so it can apply the activation itself."""
+    value next to its up value, so it can apply the activation itself.
 
-    def __init__(self, prefix: str, runtime: Runtime, *, hidden_size: int, intermediate_size: int) -> None:
+    ``rule = (steepness, limit, up_shift)`` makes it another gated unit: with ``g = min(gate(x),
+    limit)`` and ``u = clamp(up(x), -limit, limit)`` where ``limit > 0``, ``down(g * sigmoid(steepness
+    * g) * (u + up_shift))``; the default ``(1, 0, 0)`` is SwiGLU.  ``names``: the three matrices'
+    tensor names under the part's prefix."""
+
+    def __init__(self, prefix: str, runtime: Runtime, *, hidden_size: int, intermediate_size: int,
+                 rule: tuple[float, float, float] = (1.0, 0.0, 0.0),
+                 names: tuple[str, str, str] = ("gate_proj.weight", "up_proj.weight", "down_proj.weight")) -> None:
         super().__init__(prefix, runtime)
         self.hidden_size = int(hidden_size)
         self.intermediate_size = int(intermediate_size)
+        self.rule = tuple(float(v) for v in rule)
+        self.gate_name, self.up_name, self.down_name = names
         self.gate_up_weight: torch.Tensor | None = None
         self.down_weight: torch.Tensor | None = None
 
     def tensor_specs(self) -> dict[str, TensorSpec]:
         return {
-            self.name("gate_proj.weight"): TensorSpec((self.intermediate_size, self.hidden_size)),
-            self.name("up_proj.weight"): TensorSpec((self.intermediate_size, self.hidden_size)),
-            self.name("down_proj.weight"): TensorSpec((self.hidden_size, self.intermediate_size)),
+            self.name(self.gate_name): TensorSpec((self.intermediate_size, self.hidden_size)),
+            self.name(self.up_name): TensorSpec((self.intermediate_size, self.hidden_size)),
+            self.name(self.down_name): TensorSpec((self.hidden_size, self.intermediate_size)),
         }
 
     def activation_bytes(self, tokens: int, itemsize: int) -> int:
@@ -37,10 +46,10 @@ class SwiGLU(FeedForward):
         return tokens * (3 * self.intermediate_size * itemsize + self.hidden_size * 4)
 
     def load(self, tensors: Mapping[str, torch.Tensor]) -> None:
-        gate, up = tensors[self.name("gate_proj.weight")], tensors[self.name("up_proj.weight")]
+        gate, up = tensors[self.name(self.gate_name)], tensors[self.name(self.up_name)]
         self.gate_up_weight = torch.stack([gate, up], dim=1).reshape(2 * gate.shape[0], gate.shape[1]).contiguous()
-        self.down_weight = tensors[self.name("down_proj.weight")].contiguous()
+        self.down_weight = tensors[self.name(self.down_name)].contiguous()
 
     def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
         ops = self.runtime.ops
-        return ops.linear(ops.linear_swiglu(x, self.gate_up_weight), self.down_weight, for_residual=True)
+        return ops.linear(ops.linear_swiglu(x, self.gate_up_weight, self.rule), self.down_weight, for_residual=True)

@@ -21,6 +21,7 @@ POSITION_ENCODINGS: dict[str, type] = {}
 BLOCKS: dict[str, type] = {}
 EMBEDDINGS: dict[str, type] = {}
 HEADS: dict[str, type] = {}
+STREAM_STEPS: dict[str, type] = {}
 
 _TABLES = {
     "mixer": MIXERS,
@@ -30,6 +31,7 @@ _TABLES = {
     "block": BLOCKS,
     "embedding": EMBEDDINGS,
     "head": HEADS,
+    "stream_step": STREAM_STEPS,
 }
 
 
@@ -71,9 +73,13 @@ def register_head(kind: str) -> Callable[[type[T]], type[T]]:
     return _register(HEADS, "head", kind)
 
 
+def register_stream_step(kind: str) -> Callable[[type[T]], type[T]]:
+    return _register(STREAM_STEPS, "stream_step", kind)
+
+
 def build_part(role: str, spec: PartSpec, prefix: str, runtime: Runtime, **extra: Any) -> Any:
     """Instantiate ``spec`` from the registry of ``role`` (``"mixer"``, ``"feed_forward"``,
-    ``"norm"``, ``"position_encoding"``, ``"block"``, ``"embedding"`` or ``"head"``)."""
+    ``"norm"``, ``"position_encoding"``, ``"block"``, ``"embedding"``, ``"head"`` or ``"stream_step"``)."""
     table = _TABLES[role]
     try:
         cls = table[spec.kind]

@@ -22,6 +22,18 @@ def rotary_tables(capacity: int, head_dim: int, theta: float, factor: float) -> 
     return angles.cos().contiguous(), angles.sin().contiguous()
 
 
+def normed_store(runtime: Runtime, qkv, num_heads, num_kv_heads, head_dim, value_dim, ctx, cache: PagedKVView, slots,
+                 head_norm: tuple | None, cos, sin):
+    """The store of a mixer that asked for more than an encoding alone does: a norm per q and k
+    head (``head_norm = (q_gain, k_gain, eps, gain_offset)``) and values of a width of their own,
+    with the rotation by ``cos``/``sin`` where given, all in one pass (``ops.head_norm_store``)."""
+    q_gain, k_gain, eps, gain_offset = head_norm if head_norm is not None else (None, None, 0.0, 0.0)
+    return runtime.ops.head_norm_store(
+        qkv, cache.k, cache.v, q_gain, k_gain, eps, ctx.positions, slots, num_heads, num_kv_heads, head_dim, value_dim,
+        cache.block_size, runtime.dtype, gain_offset=gain_offset, cos=cos, sin=sin, max_position=ctx.max_context_len - 1,
+    )
+
+
 @register_position_encoding("rope")
 class RotaryEncoding(PositionEncoding):
     """Half-split rotary encoding: the pair ``(i, i + D/2)`` of every query and key head is
@@ -78,9 +90,13 @@ class RotaryEncoding(PositionEncoding):
         self.sin = sin.to(self.runtime.device)
         self.capacity = target
 
-    def encode_and_store(self, qkv, num_heads, num_kv_heads, head_dim, ctx, cache: PagedKVView):
+    def encode_and_store(self, qkv, num_heads, num_kv_heads, head_dim, ctx, cache: PagedKVView, *,
+                         value_dim: int | None = None, head_norm: tuple | None = None):
         self.ensure_capacity(ctx.max_context_len)
         slots = ctx.slot_mapping[cache.group] if cache.writable else None
+        if head_norm is not None or (value_dim is not None and value_dim != head_dim):
+            return normed_store(self.runtime, qkv, num_heads, num_kv_heads, head_dim, value_dim or head_dim, ctx, cache,
+                                slots, head_norm, self.cos, self.sin)
         return self.runtime.ops.rope_store(
             qkv, cache.k, cache.v, self.cos, self.sin, ctx.positions, slots,
             num_heads, num_kv_heads, head_dim, cache.block_size, ctx.max_context_len - 1, self.runtime.dtype,
@@ -96,8 +112,12 @@ class NoPositionEncoding(PositionEncoding):
     def __init__(self, prefix: str, runtime: Runtime) -> None:
         super().__init__(prefix, runtime)
 
-    def encode_and_store(self, qkv, num_heads, num_kv_heads, head_dim, ctx, cache: PagedKVView):
+    def encode_and_store(self, qkv, num_heads, num_kv_heads, head_dim, ctx, cache: PagedKVView, *,
+                         value_dim: int | None = None, head_norm: tuple | None = None):
         slots = ctx.slot_mapping[cache.group] if cache.writable else None
+        if head_norm is not None or (value_dim is not None and value_dim != head_dim):
+            return normed_store(self.runtime, qkv, num_heads, num_kv_heads, head_dim, value_dim or head_dim, ctx, cache,
+                                slots, head_norm, None, None)
         return self.runtime.ops.rope_store(
             qkv, cache.k, cache.v, None, None, ctx.positions, slots,
             num_heads, num_kv_heads, head_dim, cache.block_size, ctx.max_context_len - 1, self.runtime.dtype,
