@@ -699,3 +699,18 @@ extern "C" int ts_stream_offset(float* residual, const float* origin, const void
     return TS_ERR_DTYPE;
   return ts_launch_status();
 }
+
+// ---------------------------------------------------------------------------------------------
+// copy of 32-bit values by a kernel (a recorded step holds kernels only, no copy nodes).
+// ---------------------------------------------------------------------------------------------
+__global__ void copy_f32_kernel(float* __restrict__ out, const float* __restrict__ in, size_t total) {
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx < total) out[idx] = in[idx];
+}
+
+extern "C" int ts_copy_f32(float* out, const float* in, long total, hipStream_t stream) {
+  if (total == 0) return TS_OK;
+  if (!out || !in || total < 0) return TS_ERR_ARG;
+  hipLaunchKernelGGL(copy_f32_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, out, in, (size_t)total);
+  return ts_launch_status();
+}

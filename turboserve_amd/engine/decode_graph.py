@@ -42,6 +42,8 @@ class _Graph:
         self.graph: torch.cuda.CUDAGraph | None = None
         self.device_ints: torch.Tensor | None = None
         self.host_ints: list[torch.Tensor] = []
+        #: Per pinned buffer: the event behind the last copy that read it (None: never copied from).
+        self.host_read: list[torch.cuda.Event | None] = [None, None]
         self.turn = 0
         self.ctx: StepContext | None = None
         self.logits: torch.Tensor | None = None
@@ -130,6 +132,11 @@ class DecodeGraphs:
         element ``j`` of a device tensor."""
         shape.turn ^= 1
         host = shape.host_ints[shape.turn]
+        # The copy that last read this buffer may still be waiting behind earlier steps (a caller
+        # that wants no logits of a step waits for nothing): it must have happened before the
+        # buffer is written again.
+        if shape.host_read[shape.turn] is not None:
+            shape.host_read[shape.turn].synchronize()
         data = host.numpy()
         pack_step(data, shape.layout, entries, range(shape.batch), pad_state_slot=self.pad_state_slot, token_sources=patch,
                   recorded=True)
@@ -152,6 +159,9 @@ class DecodeGraphs:
             shape = self._graphs[key] = self._build(key)
         host = self._fill(shape, entries, tokens_from[1] if tokens_from else None, check=check)
         shape.device_ints.copy_(host, non_blocking=True)
+        if shape.host_read[shape.turn] is None:
+            shape.host_read[shape.turn] = torch.cuda.Event()
+        shape.host_read[shape.turn].record(torch.cuda.current_stream(self.device))
         if tokens_from and tokens_from[1]:
             self.model.runtime.ops.patch_tokens(shape.ctx.token_ids, shape.ctx.token_source, tokens_from[0])
         shape.graph.replay()

@@ -56,6 +56,7 @@ _SIGNATURES: dict[str, dict[str, list]] = {
                                c_float, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
                                c_int, c_int, c_int, c_void_p],
         "ts_embed_positions": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+        "ts_copy_f32": [c_void_p, c_void_p, c_long, c_void_p],
         "ts_stream_offset": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
         "ts_moe_route": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
                          c_int, c_float, c_int, c_void_p],
@@ -509,6 +510,15 @@ class Ops:
         out = torch.empty((tokens, hidden), dtype=torch.float32, device=table.device)
         _check(self.core.ts_embed_positions(_ptr(out), _ptr(table), _ptr(ids), _ptr(positions), _ptr(at), tokens, hidden,
                                             vocab, dtype_code(table.dtype), self.stream()), "ts_embed_positions")
+        return out
+
+    def copy_float32(self, x: torch.Tensor) -> torch.Tensor:
+        """A copy of a contiguous 32-bit tensor made by a kernel: a step that is recorded holds
+        kernels only, and torch's ``clone`` would record a copy node."""
+        _gpu(x)
+        _need(x.dtype == torch.float32 and x.is_contiguous(), "x must be contiguous float32")
+        out = torch.empty_like(x)
+        _check(self.core.ts_copy_f32(_ptr(out), _ptr(x), x.numel(), self.stream()), "ts_copy_f32")
         return out
 
     def stream_offset(self, residual: torch.Tensor, origin: torch.Tensor | None, offset: torch.Tensor | None) -> None:

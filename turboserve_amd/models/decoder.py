@@ -189,7 +189,7 @@ class DecoderModel:
             raise ValueError(f"{len(caches)} cache views for {len(self.plan.schedule)} scheduled layer calls")
         stream = ResidualStream(self.embedding.forward(token_ids, ctx))
         # The embedding's output is kept apart only where a stream step adds it in again later.
-        origin = stream.residual.clone() if self.keeps_origin else None
+        origin = self.runtime.ops.copy_float32(stream.residual) if self.keeps_origin else None
         for call, cache, enter in zip(self.plan.schedule, caches, self.enter_steps):
             if enter is not None:
                 stream = enter.forward(stream, ctx, origin)
