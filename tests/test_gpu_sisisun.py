@@ -1,0 +1,312 @@
+"""Sisisun on the GPU against the plain implementation (``tests/plain/sisisun_plain.py``): each
+mechanism's kernel alone, whole prompts, every way of cutting requests into steps on so few
+pages that they are used again, a key far back that one query rests on, and greedy generation
+through the engine's own entry point."""
+
+from __future__ import annotations
+
+import copy
+
+import pytest
+import torch
+
+import sisisun_tiny as st
+import trace_helpers as th
+from plain import sisisun_plain as plain
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+#: 32-bit engine against the 32-bit plain implementation, relative to a position's largest logit.
+RTOL_F32 = 2e-4
+#: bfloat16 engine (weights stored in bfloat16) against the plain implementation in 32-bit on the
+#: same weights.
+RTOL_BF16 = 4e-2
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from turboserve_amd.kernels.ops import Ops
+
+    return Ops(DEV)
+
+
+def excess(got: torch.Tensor, want: torch.Tensor, dtype: str) -> float:
+    """The largest |difference| of a position's logits over the bound for that position."""
+    rtol = RTOL_F32 if dtype == "float32" else RTOL_BF16
+    bound = rtol * want.abs().amax(dim=-1, keepdim=True).clamp_min(1.0)
+    return float(((got - want).abs() / bound).max())
+
+
+# ---------------------------------------------------------------------------------------------
+# mechanisms alone
+# ---------------------------------------------------------------------------------------------
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("hidden", [52, 256, 4100])
+def test_norm_with_a_gain_around_zero(ops, dtype, hidden):
+    g = torch.Generator().manual_seed(hidden)
+    residual = torch.randn(5, hidden, generator=g) * 3
+    pending = torch.randn(5, hidden, generator=g).to(dtype)
+    gain = (0.3 * torch.randn(hidden, generator=g)).to(dtype)
+    want_sum = residual + pending.float()
+    want = plain.unit_gain_norm(want_sum, gain.float(), 1e-5)
+    stream = residual.clone().to(DEV)
+    got = ops.add_rmsnorm(stream, pending.to(DEV), gain.to(DEV), 1e-5, gain_offset=1.0, one_rounding=True)
+    assert torch.allclose(stream.cpu(), want_sum, atol=1e-6)
+    tol = dict(rtol=1e-5, atol=1e-5) if dtype == torch.float32 else dict(rtol=1e-2, atol=1e-2)
+    torch.testing.assert_close(got.float().cpu(), want, **tol)
+    rows = torch.tensor([3, 0], dtype=torch.int32, device=DEV)
+    picked = ops.add_rmsnorm(stream, None, gain.to(DEV), 1e-5, rows, gain_offset=1.0, one_rounding=True)
+    torch.testing.assert_close(picked.float().cpu(), want[[3, 0]], **tol)
+    alone = ops.rmsnorm(want_sum.to(dtype).to(DEV), gain.to(DEV), 1e-5, gain_offset=1.0, one_rounding=True)
+    torch.testing.assert_close(alone.float().cpu(), plain.unit_gain_norm(want_sum.to(dtype).float(), gain.float(), 1e-5), **tol)
+
+
+def test_token_rows_plus_position_vectors(ops):
+    from turboserve_amd.parts.ends import sinusoid_table
+
+    g = torch.Generator().manual_seed(1)
+    table = torch.randn(30, 14, generator=g)
+    ids = [4, 29, 0, 7, 7]
+    positions = [0, 1, 2, 1000, 3999]
+    at = sinusoid_table(4000, 14, 10000.0).to(DEV)
+    got = ops.embed_positions(table.to(DEV), torch.tensor(ids, dtype=torch.int32, device=DEV),
+                              torch.tensor(positions, dtype=torch.int32, device=DEV), at).cpu()
+    want = table[ids] + plain.sinusoid_rows(positions, 14)
+    torch.testing.assert_close(got, want, rtol=0, atol=2e-6)
+
+
+def test_stream_offsets(ops):
+    g = torch.Generator().manual_seed(2)
+    residual, origin, offset = torch.randn(7, 20, generator=g), torch.randn(7, 20, generator=g), torch.randn(20, generator=g)
+    for with_origin in (False, True):
+        stream = residual.clone().to(DEV)
+        ops.stream_offset(stream, origin.to(DEV) if with_origin else None, offset.to(DEV))
+        torch.testing.assert_close(stream.cpu(), residual + (origin if with_origin else 0) + offset, rtol=0, atol=1e-6)
+    torch.testing.assert_close(ops.copy_float32(origin.to(DEV)).cpu(), origin, rtol=0, atol=0)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("inter", [5, 44, 96])
+def test_the_clamped_gated_unit(ops, dtype, inter):
+    g = torch.Generator().manual_seed(inter)
+    gate, up = (3 * torch.randn(9, inter, generator=g)).to(dtype), (3 * torch.randn(9, inter, generator=g)).to(dtype)
+    eye = torch.eye(inter)
+    want = plain.clamped_glu(torch.zeros(1, inter), {"p.gate": eye, "p.up": eye, "p.down": eye}, "p", 1.25)  # shape only
+    gl, ul = gate.float().clamp(max=1.25), up.float().clamp(-1.25, 1.25)
+    want = gl * torch.sigmoid(1.702 * gl) * (ul + 1)
+    paired = torch.stack([gate, up], dim=2).reshape(9, 2 * inter).contiguous()
+    got = ops.swiglu(paired.to(DEV), paired=True, rule=(1.702, 1.25, 1.0)).float().cpu()
+    tol = dict(rtol=1e-5, atol=1e-5) if dtype == torch.float32 else dict(rtol=1e-2, atol=1e-2)
+    torch.testing.assert_close(got, want, **tol)
+    plain_rule = ops.swiglu(paired.to(DEV), paired=True).float().cpu()
+    torch.testing.assert_close(plain_rule, gate.float() * torch.sigmoid(gate.float()) * up.float(), **tol)
+
+
+@pytest.mark.parametrize("experts, top, groups, keep", [(8, 2, 4, 2), (6, 1, 1, 1), (5, 3, 5, 3), (12, 3, 3, 2), (16, 3, 2, 1),
+                                                          (64, 6, 8, 3), (7, 7, 1, 1)])
+def test_the_router_takes_what_the_rule_says(ops, experts, top, groups, keep):
+    g = torch.Generator().manual_seed(experts * 31 + top)
+    hidden, tokens = 40, 50
+    x = torch.randn(tokens, hidden, generator=g)
+    router = torch.randn(experts, hidden, generator=g) * 0.4
+    extra = torch.randn(hidden, generator=g) * 0.3
+    taken, weights, gate = ops.moe_route(x.to(DEV), router.to(DEV), top=top, groups=groups, keep=keep, scale=1.7,
+                                         extra=extra.to(DEV))
+    scores = torch.sigmoid(x @ router.T)
+    for t in range(tokens):
+        want = plain.route(scores[t].tolist(), top, groups, keep)
+        assert taken[t].tolist() == want, (t, taken[t].tolist(), want)
+        chosen = scores[t, want]
+        torch.testing.assert_close(weights[t].cpu(), chosen / (chosen.sum() + 1e-20) * 1.7, rtol=1e-5, atol=1e-6)
+    torch.testing.assert_close(gate.cpu(), torch.sigmoid(x @ extra), rtol=1e-5, atol=1e-6)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_experts_pair_by_pair_and_their_weighted_sum(ops, dtype):
+    g = torch.Generator().manual_seed(9)
+    tokens, hidden, inter, experts, top = 11, 40, 24, 5, 2
+    x = torch.randn(tokens, hidden, generator=g).to(dtype)
+    gate_w = (0.3 * torch.randn(experts, inter, hidden, generator=g)).to(dtype)
+    up_w = (0.3 * torch.randn(experts, inter, hidden, generator=g)).to(dtype)
+    down_w = (0.3 * torch.randn(experts, hidden, inter, generator=g)).to(dtype)
+    taken = torch.stack([torch.randperm(experts, generator=g)[:top] for _ in range(tokens)]).to(torch.int32)
+    weights = torch.rand(tokens, top, generator=g)
+    shared = torch.randn(tokens, hidden, generator=g).to(dtype)
+    shared_gate = torch.rand(tokens, generator=g)
+    stacked = torch.stack([gate_w, up_w], dim=2).reshape(experts, 2 * inter, hidden).contiguous()
+    units = ops.moe_expert_units(x.to(DEV), stacked.to(DEV), taken.to(DEV), (1.0, 0.0, 0.0))
+    outputs = ops.moe_expert_outputs(units, down_w.to(DEV), taken.to(DEV))
+    got = ops.moe_combine(outputs, weights.to(DEV), shared.to(DEV), shared_gate.to(DEV), dtype)[0].cpu()
+    want = torch.zeros(tokens, hidden)
+    for t in range(tokens):
+        for j in range(top):
+            e = int(taken[t, j])
+            tensors = {"p.gate": gate_w[e].float(), "p.up": up_w[e].float(), "p.down": down_w[e].float()}
+            want[t] += weights[t, j] * plain.silu_glu(x[t:t + 1].float(), tensors, "p")[0]
+        want[t] += shared_gate[t] * shared[t].float()
+    tol = dict(rtol=1e-4, atol=1e-4) if dtype == torch.float32 else dict(rtol=3e-2, atol=3e-2)
+    torch.testing.assert_close(got, want, **tol)
+
+
+# ---------------------------------------------------------------------------------------------
+# models
+# ---------------------------------------------------------------------------------------------
+
+
+def lengths_for(name: str) -> list[int]:
+    return {"P": [1, 9, 40, 75, 66, 130], "Q": [2, 17, 33, 70, 50], "R": [3, 45, 97, 200, 64]}[name]
+
+
+@pytest.fixture(scope="module", params=["P", "Q", "R"])
+def case(request, tmp_path_factory):
+    name = request.param
+    config, seed, page = st.TINY[name]
+    folders = {
+        "float32": st.make_model_dir(tmp_path_factory.mktemp(f"sisisun{name}_f32"), config, seed, torch.float32, std=0.15),
+        "bfloat16": st.make_model_dir(tmp_path_factory.mktemp(f"sisisun{name}_bf16"), config, seed, torch.bfloat16, std=0.08),
+    }
+    requests = {f"r{i}": st_tokens(config["vocab"], n, 300 + i) for i, n in enumerate(lengths_for(name))}
+    expected = {d: {rid: st.plain_logits(folders[d], toks) for rid, toks in requests.items()} for d in folders}
+    return {"name": name, "page": page, "folders": folders, "requests": requests, "expected": expected}
+
+
+def st_tokens(vocab: int, length: int, seed: int) -> list[int]:
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(0, vocab, (length,), generator=g).tolist()
+
+
+def run_trace(folder, dtype: str, page: int, steps: list[dict], max_tokens: int | None = None):
+    from turboserve_amd.engine.replay import TraceReplayer
+
+    replayer = TraceReplayer(folder, dtype=dtype, max_tokens=max_tokens or th.peak_tokens(steps, rounding=page), page_size=page)
+    outputs = {}
+    for record in steps:
+        logits = replayer.run_step(record)
+        if logits.shape[0]:
+            outputs[record["step"]] = logits.float().cpu()
+    replayer.manager.check_invariants()
+    assert all(pool.num_in_use == 0 for pool in replayer.manager.pools), "pages were not given back"
+    return outputs
+
+
+def check_against_plain(case, dtype: str, steps: list[dict]) -> None:
+    outputs = run_trace(case["folders"][dtype], dtype, case["page"], steps)
+    got = th.collect(steps, outputs, case["requests"])
+    for rid, want in case["expected"][dtype].items():
+        worst = excess(got[rid], want, dtype)
+        assert worst <= 1.0, f"{case['name']} {dtype} {rid}: {worst:.2f} times the bound"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_whole_prompts(case, dtype):
+    check_against_plain(case, dtype, th.whole(case["requests"]))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_prefix_then_token_by_token(case, dtype):
+    check_against_plain(case, dtype, th.prefix_then_single(case["requests"], tail=40))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("sizes", [(2, 3, 5, 2, 16, 7), (33, 2, 17, 64), (1, 2)])
+def test_portions_of_changing_size(case, dtype, sizes):
+    check_against_plain(case, dtype, th.portions(case["requests"], sizes))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_mixed_batches_on_pages_that_are_used_again(case, dtype):
+    steps = th.mixed(case["requests"], (7, 2, 19, 32, 3), max_live=3, decode_tail=9)
+    check_against_plain(case, dtype, steps)
+
+
+def test_cuttings_agree_in_32_bit(case):
+    """The logits of a position do not depend on how its request was cut or batched."""
+    folder, page = case["folders"]["float32"], case["page"]
+    ways = {"whole": th.whole(case["requests"]), "single": th.prefix_then_single(case["requests"], tail=40),
+            "portions": th.portions(case["requests"], (2, 5, 3, 24)), "mixed": th.mixed(case["requests"], (5, 2, 21), max_live=4)}
+    results = {name: th.collect(steps, run_trace(folder, "float32", page, steps), case["requests"]) for name, steps in ways.items()}
+    for name, got in results.items():
+        for rid, base in results["whole"].items():
+            scale = base.abs().amax(dim=-1, keepdim=True).clamp_min(1.0)
+            assert float(((got[rid] - base).abs() / scale).max()) <= 2e-5, (name, rid)
+
+
+# ---------------------------------------------------------------------------------------------
+# one key far back
+# ---------------------------------------------------------------------------------------------
+
+FAR_CONFIG = {
+    "architecture": "Sisisun", "vocab": 64, "width": 64, "norm": {"eps": 1e-6},
+    "layers": [st.layer(st.attention(2, 2, 32, 32, 9.0, scale=1.0), None), st.layer(st.attention(2, 1, 32, 16, 9.0, scale=1.0), st.dense(64, 2.0))],
+    "loop": {"start": 0, "stop": 1, "times": 2},
+}
+MARK, ASKS = 7, 9  # the token far back and the token whose query looks for it
+
+
+def far_model(folder, dtype: torch.dtype):
+    """Weights under which the query of token ASKS puts most of its weight on the key of token
+    MARK wherever that lies: both tokens share a large row of the table, and the first layer's
+    keys are made by the matrix that makes its queries, so their directions agree."""
+    tensors = st.draw_tensors(FAR_CONFIG, 21, torch.float32, 0.12)
+    direction = torch.randn(64, generator=torch.Generator().manual_seed(3))
+    tensors["embed"][MARK] = 5.0 * direction
+    tensors["embed"][ASKS] = 5.0 * direction + tensors["embed"][ASKS] * 0.2
+    tensors["l0.mix.k"] = tensors["l0.mix.q"].clone()
+    tensors["l0.mix.k.norm"] = tensors["l0.mix.q.norm"].clone()
+    tensors["l0.mix.v"] = tensors["l0.mix.v"] * 4.0
+    tensors = {name: t.to(dtype).contiguous() for name, t in tensors.items()}
+    return st.make_model_dir(folder, FAR_CONFIG, 0, tensors=tensors)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("mark_at", [0, 1, 15, 16, 17, 127, 128, 250])
+def test_a_key_far_back_is_found(tmp_path, dtype, mark_at):
+    folder = far_model(tmp_path / "far", torch.float32 if dtype == "float32" else torch.bfloat16)
+    config, tensors = st.read_model_dir(folder)
+    length = 300
+    filler = [t for t in st_tokens(64, 2 * length, 77) if t not in (MARK, ASKS)][:length]
+    tokens = list(filler)
+    tokens[mark_at] = MARK
+    tokens[-1] = ASKS
+    tokens[-20] = ASKS
+    want = plain.forward(config, tensors, tokens)
+    without = list(tokens)
+    without[mark_at] = filler[mark_at]
+    moved = (plain.forward(config, tensors, without)[-1] - want[-1]).abs().max() / want[-1].abs().max()
+    assert moved > 0.1, f"the far key does not matter enough to this model's last logits ({float(moved):.3f})"
+    requests = {"far": tokens}
+    for steps in (th.whole(requests), th.prefix_then_single(requests, tail=30), th.portions(requests, (17, 2, 64, 5))):
+        got = th.collect(steps, run_trace(folder, dtype, 16, steps), requests)["far"]
+        rows = [length - 20, length - 1]
+        assert excess(got[rows], want[rows], dtype) <= 1.0
+
+
+# ---------------------------------------------------------------------------------------------
+# generation through the engine
+# ---------------------------------------------------------------------------------------------
+
+
+@pytest.mark.parametrize("name", ["P", "Q"])
+def test_greedy_generation_through_the_engine(tmp_path, name):
+    from turboserve_amd.config.engine_config import EngineConfig, SchedulerConfig
+    from turboserve_amd.engine.llm_engine import LLMEngine
+    from turboserve_amd.sampling.params import SamplingParams
+
+    config, seed, page = st.TINY[name]
+    folder = st.make_model_dir(tmp_path / "gen", config, seed + 5, torch.float32, std=0.2)
+    raw, tensors = st.read_model_dir(folder)
+    prompts = [st_tokens(config["vocab"], n, 900 + n) for n in (3, 21, 1, 50)]
+    new = 40
+    want = [st.greedy(raw, tensors, prompt, new) for prompt in prompts]
+    engine = LLMEngine(EngineConfig(
+        model=str(folder), dtype="float32",
+        scheduler=SchedulerConfig(max_num_seqs=4, max_num_batched_tokens=64, block_size=page, num_blocks=40),
+    ))
+    outputs = engine.generate(prompts, SamplingParams(max_tokens=new, temperature=0.0, ignore_eos=True))
+    assert [out.new_token_ids for out in outputs] == want
+    # Once more on the same engine: the pages and slots of the first round are used again.
+    again = engine.generate(list(reversed(prompts)), SamplingParams(max_tokens=new, temperature=0.0, ignore_eos=True))
+    assert [out.new_token_ids for out in again] == list(reversed(want))
