@@ -33,7 +33,7 @@ and one 2,048-token prompt), ``--shape 32b --batch 64 --fill-hbm`` (a cache pool
 free memory), ``--closed-loop C [--sampled]`` (the reference's serving profile driven offline: 256
 requests of 128..1,024 tokens in and 64..512 out, C in flight; the library's products run at a
 few step sizes that are all timed at start-up, about 70 s the first time), ``--attention-prefill T[,CTX]`` (the
-prefill attention kernel alone), ``--sample-kernel ROWS`` (the sampling kernel alone), ``--hbm-read`` (a kernel that only reads: what the memory gives), ``--only-prefill [TOKENS]`` (one prompt's prefill alone, 2,048 tokens or TOKENS), ``--kernel-shares TRACE.csv`` (no GPU: the per-kernel table of a
+prefill attention kernel alone), ``--sample-kernel ROWS`` (the sampling kernel alone), ``--hbm-read`` (a kernel that only reads: what the memory gives), ``--only-prefill [TOKENS]`` (one prompt's prefill alone, 2,048 tokens or TOKENS), ``--designs [2k,4k]`` (the Sisisun design beside a Qwen2 model of equal layer sizes: prefill and decode), ``--kernel-shares TRACE.csv`` (no GPU: the per-kernel table of a
 ``rocprofv3 --kernel-trace`` of any of these runs).
 """
 
@@ -120,6 +120,10 @@ def parse_args(argv: list[str] | None = None) -> argparse.Namespace:
     p.add_argument("--attention-prefill", metavar="TOKENS[,CONTEXT]", default=None,
                    help="time the prefill attention kernel alone on the shape's heads: one request that brings TOKENS "
                         "tokens and holds CONTEXT afterwards (default: TOKENS), and exit")
+    p.add_argument("--designs", nargs="?", const="2k,4k", default=None, metavar="SIZES",
+                   help="prefill and decode of the Sisisun design (random weights) at layer sizes that resemble a real "
+                        "model's (2k, 4k: the width), beside a Qwen2 model of the same width, heads, feed-forward and "
+                        "number of layer runs; prints one JSON object and exits")
     return p.parse_args(argv)
 
 
@@ -475,6 +479,85 @@ def run_hbm_read(launches: int = 12) -> dict:
             "best": max(table.values()), "peak": HBM_PEAK_GBS}
 
 
+#: ``--designs``: per size the Sisisun configuration and the Qwen2 configuration it is set beside.  Both have the same
+#: width, heads, head size, dense feed-forward, vocabulary and number of layer runs; every second Sisisun layer is routed.
+def design_pair(size: str) -> tuple[dict, dict]:
+    width, heads, kv, ff, experts, top, expert_ff, shared_ff = {
+        "2k": (2048, 16, 4, 8192, 32, 4, 1024, 2048),
+        "4k": (4096, 32, 8, 14336, 64, 6, 1408, 2816),
+    }[size]
+    mixer = {"heads": heads, "kv_heads": kv, "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "softcap": 30.0}
+    dense = {"kind": "dense", "ff": ff, "limit": 7.0}
+    routed = {"kind": "moe", "expert": {"ff": expert_ff}, "shared": {"ff": shared_ff},
+              "router": {"experts": experts, "top": top, "scale": 2.5, "groups": {"count": 8, "keep": 4}}}
+    layers = [{"type": "attention", "mixer": mixer, "mlp": dense if i % 2 == 0 else routed} for i in range(6)]
+    sisisun = {"architecture": "Sisisun", "vocab": 32000, "width": width, "norm": {"eps": 1e-6}, "layers": layers,
+               "loop": {"start": 0, "stop": 2, "times": 2}}
+    qwen2 = dict(SHAPE_7B, hidden_size=width, num_hidden_layers=8, num_attention_heads=heads, num_key_value_heads=kv,
+                 head_dim=128, intermediate_size=ff, vocab_size=32000)
+    return sisisun, qwen2
+
+
+def active_weight_elements(model, batch: int) -> float:
+    """Elements of the weights a step of ``batch`` tokens reads: every tensor of every layer run
+    once, but of a routed feed-forward's experts only as many as ``batch`` tokens can take."""
+    from turboserve_amd.parts.experts import RoutedExperts
+
+    total = 0.0
+    for call in model.plan.schedule:
+        block = model.blocks[call.layer]
+        forward = getattr(block, "feed_forward", None)
+        for name, spec in block.tensor_specs().items():
+            count = 1
+            for dim in spec.shape:
+                count *= dim
+            if isinstance(forward, RoutedExperts) and name.startswith(forward._expert(0, 1).rsplit("e0", 1)[0] + "e"):
+                count *= min(1.0, batch * forward.top / forward.experts)
+            total += count
+    head = model.plan.vocab_size * model.plan.hidden_size
+    return total + head
+
+
+def run_designs(sizes: list[str], dtype_name: str, steps: int, warmup: int) -> dict:
+    """Prefill (2,048 tokens, best of three) and decode (8 requests at 2,048 tokens of context)
+    of both designs at each size, through ``LLMEngine``; with the bytes a decode step reads and
+    the multiply-adds a prompt takes, so that both can be set against what the device gives."""
+    import torch
+
+    from turboserve_amd.engine.loading import build_model, make_runtime, resolve_run_dtype
+    from turboserve_amd.weights.random_init import random_tensors_on_device
+
+    dtype = resolve_run_dtype(dtype_name)
+    itemsize = 2 if dtype == torch.bfloat16 else 4
+    peak = PEAK_FLOPS["bf16" if dtype == torch.bfloat16 else "fp32"]
+    batch, context, prompt = 8, 2048, 2048
+    out: dict = {"dtype": dtype_name, "decode": f"{batch} requests at {context} tokens", "prefill": f"{prompt} tokens"}
+    for size in sizes:
+        for label, shape in zip(("sisisun", "qwen2"), design_pair(size)):
+            runtime = make_runtime(dtype, "cuda:0")
+            config, model = build_model(shape, runtime)
+            random_tensors_on_device(model, seed=0)
+            seconds = run_prefill(model, config, prompt, tune=False)
+            decode = run_decode(model, config, batch, context - 1, steps=steps, warmup=warmup)
+            needs = [need for need in model.cache_needs() if need is not None]
+            kv_elements = sum(n.num_kv_heads * (n.head_dim + n.value_width) for n in needs)
+            read = (active_weight_elements(model, batch) + batch * decode["mean_context"] * kv_elements) * itemsize
+            attention = sum(4.0 * prompt * prompt / 2 * (n.head_dim + n.value_width) / 2 for n in needs)  # causal
+            heads_per_kv = [model.blocks[c.layer].mixer.num_heads // model.blocks[c.layer].mixer.num_kv_heads for c in model.plan.schedule]
+            flops = 2.0 * prompt * (active_weight_elements(model, prompt) - model.plan.vocab_size * model.plan.hidden_size) \
+                + sum(4.0 * prompt * prompt / 2 * n.num_kv_heads * g * (n.head_dim + n.value_width) / 2 for n, g in zip(needs, heads_per_kv))
+            out[f"{size}_{label}"] = {
+                "layer_runs": len(model.plan.schedule), "parameters_M": round(model.num_parameters() / 1e6, 1),
+                "prefill_ms": round(seconds * 1e3, 3), "prefill_tokens_per_s": round(prompt / seconds, 1),
+                "prefill_flops_frac": round(flops / seconds / peak, 4),
+                "decode_ms_per_step": round(decode["step_seconds"] * 1e3, 4), "decode_tokens_per_s": round(decode["tokens_per_s"], 1),
+                "decode_read_GB": round(read / 1e9, 4), "decode_hbm_frac": round(read / decode["step_seconds"] / 1e9 / HBM_PEAK_GBS, 4),
+            }
+            del model, runtime
+            torch.cuda.empty_cache()
+    return out
+
+
 def decode_bytes(config, layers: int, batch: int, context: float, itemsize: int) -> float:
     """Bytes a decode step has to read: every weight it uses once (all but the embedding
     table, of which it reads one row per request) and the cache of the live requests."""
@@ -512,6 +595,9 @@ def main(argv: list[str] | None = None) -> int:
     if args.attention_prefill:
         sizes = [int(v) for v in args.attention_prefill.split(",")]
         print(json.dumps(run_attention_prefill(SHAPES[args.shape][1], sizes[0], sizes[-1])))
+        return 0
+    if args.designs:
+        print(json.dumps(run_designs(args.designs.split(","), args.dtype, min(args.steps, 32), min(args.warmup, 8))))
         return 0
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this engine (single-GPU by design)")

@@ -265,6 +265,27 @@ __device__ __forceinline__ f32x4 score_tile(const KeyFrags& f, int t, const Quer
   return s;
 }
 
+// How a raw score (q . k) becomes the exponent of its weight: with cap > 0 it is first bent to
+// cap * tanh(raw / cap) (cap is in units of raw scores: the softcap of the scaled scores over the
+// scale), then multiplied by k = scale * log2(e).
+struct ScoreRule {
+  float k;
+  float cap;
+  float inv_cap;
+};
+
+static inline ScoreRule score_rule(float scale, float softcap) {
+  const float cap = softcap > 0.f ? softcap / scale : 0.f;
+  return ScoreRule{scale * 1.4426950408889634f, cap, cap > 0.f ? 1.f / cap : 0.f};
+}
+
+__device__ __forceinline__ float capped(float raw, ScoreRule rule) {
+  if (rule.cap <= 0.f) return raw;
+  // tanh(x) = 1 - 2 / (2^(2 x log2 e) + 1); exact at both ends (2^inf = inf, 2^-inf = 0).
+  const float e = __builtin_amdgcn_exp2f(raw * rule.inv_cap * 2.8853900817779268f);
+  return rule.cap * (1.f - 2.f * __builtin_amdgcn_rcpf(e + 1.f));
+}
+
 // Online-softmax state of the lane's column.
 struct ColumnState {
   float m;  // running maximum of the scaled scores (log2 domain)
@@ -286,12 +307,12 @@ __device__ __forceinline__ void init_state(ColumnState& st) {
 // that every key of the window is visible to every column of the wavefront.
 template <bool MASKED>
 __device__ __forceinline__ Frag8 softmax_window(ColumnState& st, const f32x4 s0, const f32x4 s1, int w, int group,
-                                                int first_valid, int last_valid, float scale_log2, float& alpha) {
+                                                int first_valid, int last_valid, ScoreRule scale_log2, float& alpha) {
   float s[8];  // unscaled scores; e = 4 t + i is row 4 g + i of tile t
   float mx = -INFINITY;
 #pragma unroll
   for (int e = 0; e < 8; ++e) {
-    const float raw = e < 4 ? s0[e & 3] : s1[e & 3];
+    const float raw = capped(e < 4 ? s0[e & 3] : s1[e & 3], scale_log2);
     if (MASKED) {
       const int key = w + 8 * group + e;
       s[e] = (key >= first_valid && key <= last_valid) ? raw : -INFINITY;
@@ -300,7 +321,7 @@ __device__ __forceinline__ Frag8 softmax_window(ColumnState& st, const f32x4 s0,
     }
     mx = fmaxf(mx, s[e]);
   }
-  mx = groups_max(mx) * scale_log2;  // the scale is positive: the maximum commutes with it
+  mx = groups_max(mx) * scale_log2.k;  // the scale is positive: the maximum commutes with it
   const float m_new = fmaxf(st.m, mx);
   // Nothing visible to this column so far: keep the state, contribute zeros.
   const float m_use = (MASKED && m_new == -INFINITY) ? 0.f : m_new;
@@ -309,7 +330,7 @@ __device__ __forceinline__ Frag8 softmax_window(ColumnState& st, const f32x4 s0,
   float sum = 0.f;
 #pragma unroll
   for (int e = 0; e < 8; ++e) {
-    pe[e] = fast_exp2(fmaf(s[e], scale_log2, -m_use));  // 0 for masked keys
+    pe[e] = fast_exp2(fmaf(s[e], scale_log2.k, -m_use));  // 0 for masked keys
     sum += pe[e];
   }
   st.l = st.l * alpha + sum;
@@ -332,7 +353,7 @@ __device__ __forceinline__ void accumulate(ColumnState& st, const ValueFrags& f,
 // One window for one set of 16 columns: scores, online softmax, O^T += V^T P^T.
 template <bool MASKED>
 __device__ __forceinline__ void attend_window(ColumnState& st, const WindowFrags& f, const QueryFrags& q, int w,
-                                              int group, int first_valid, int last_valid, float scale_log2) {
+                                              int group, int first_valid, int last_valid, ScoreRule scale_log2) {
   const f32x4 s0 = score_tile(f, 0, q);
   const f32x4 s1 = score_tile(f, 1, q);
   float alpha;
@@ -342,7 +363,7 @@ __device__ __forceinline__ void attend_window(ColumnState& st, const WindowFrags
 
 // Dispatch on a wavefront-uniform flag: `interior` windows need no masks.
 __device__ __forceinline__ void attend(ColumnState& st, const WindowFrags& f, const QueryFrags& q, int w, int group,
-                                       int first_valid, int last_valid, float scale_log2, bool interior) {
+                                       int first_valid, int last_valid, ScoreRule scale_log2, bool interior) {
   if (interior)
     attend_window<false>(st, f, q, w, group, first_valid, last_valid, scale_log2);
   else
@@ -362,7 +383,7 @@ decode_kernel(float* __restrict__ partial_acc, float* __restrict__ partial_ml,
               const uint16_t* __restrict__ q, long q_stride, const uint16_t* __restrict__ k_pages,
               const uint16_t* __restrict__ v_pages, const int* __restrict__ block_table, int table_width,
               const int* __restrict__ query_start_loc, const int* __restrict__ context_lens,
-              int seq_begin, int heads, int kv_heads, int block_shift, float scale_log2, int window,
+              int seq_begin, int heads, int kv_heads, int block_shift, ScoreRule scale_log2, int window,
               int keys_per_split, int splits, const int* __restrict__ max_context) {
   // A recorded launch serves growing contexts: the longest context of the step is then read
   // from device memory and the keys are divided evenly over the fixed number of splits.
@@ -524,7 +545,7 @@ prefill_kernel(uint16_t* __restrict__ out, const uint16_t* __restrict__ q, long 
                const uint16_t* __restrict__ k_pages, const uint16_t* __restrict__ v_pages,
                const int* __restrict__ block_table, int table_width, const int* __restrict__ query_start_loc,
                const int* __restrict__ context_lens, const int* __restrict__ blocks, int heads, int kv_heads,
-               int block_shift, float scale_log2, int window) {
+               int block_shift, ScoreRule scale_log2, int window) {
   const int lane = threadIdx.x;
   const int lane16 = lane & 15;
   const int group = lane >> 4;
@@ -737,7 +758,7 @@ prefill_shared_kernel(uint16_t* __restrict__ out, const uint16_t* __restrict__ q
                       const uint16_t* __restrict__ k_pages, const uint16_t* __restrict__ v_pages,
                       const int* __restrict__ block_table, int table_width, const int* __restrict__ query_start_loc,
                       const int* __restrict__ context_lens, const int* __restrict__ blocks, int num_blocks,
-                      int pair_blocks, int heads, int kv_heads, int block_shift, float scale_log2, int window) {
+                      int pair_blocks, int heads, int kv_heads, int block_shift, ScoreRule scale_log2, int window) {
   extern __shared__ __attribute__((aligned(16))) uint16_t staged[];  // [2][K_TILE] then [2][V_TILE]
   uint16_t* ks = staged;
   uint16_t* vs = staged + 2 * K_TILE;
@@ -868,7 +889,7 @@ static int launch_prefill_shared(hipStream_t stream, uint16_t* out, const uint16
                                  const uint16_t* k_pages, const uint16_t* v_pages, const int* block_table,
                                  int table_width, const int* query_start_loc, const int* context_lens,
                                  const int* blocks, int num_blocks, int heads, int kv_heads, int shift,
-                                 float scale_log2, int window) {
+                                 ScoreRule scale_log2, int window) {
   constexpr size_t lds = (size_t)2 * (K_TILE + V_TILE) * sizeof(uint16_t);
   static_assert(lds <= 160 * 1024, "the staged windows must fit in LDS");
   if (lds > 48 * 1024) {
@@ -1120,7 +1141,7 @@ prefill_wide_kernel(uint16_t* __restrict__ out, const uint16_t* __restrict__ q, 
                     const uint16_t* __restrict__ k_pages, const uint16_t* __restrict__ v_pages,
                     const int* __restrict__ block_table, int table_width, const int* __restrict__ query_start_loc,
                     const int* __restrict__ context_lens, const int* __restrict__ blocks, int num_blocks,
-                    int pair_blocks, int group_heads, int heads, int kv_heads, int block_shift, float scale_log2,
+                    int pair_blocks, int group_heads, int heads, int kv_heads, int block_shift, ScoreRule scale_log2,
                     int window, const int* __restrict__ ranges, float* __restrict__ partial_acc,
                     float* __restrict__ partial_ml) {
   extern __shared__ __attribute__((aligned(16))) uint16_t staged[];  // [2][K_TILE] then [2][V_TILE]
@@ -1287,6 +1308,10 @@ prefill_wide_kernel(uint16_t* __restrict__ out, const uint16_t* __restrict__ q, 
   auto look = [&](auto parity, auto steady, int w) __attribute__((always_inline)) {
     constexpr int A = decltype(parity)::value;
     constexpr int B = A ^ 1;
+    if (scale_log2.cap > 0.f) {
+#pragma unroll
+      for (int e = 0; e < 16; ++e) s[A][e] = capped(s[A][e], scale_log2);
+    }
     if (!decltype(steady)::value && !interior(w)) {
       asm volatile("" ::: "memory");  // keeps this a branch: as selects it would cost every window 64 instructions
       wide_mask(s[A], w, half, lo_col, p_col);
@@ -1299,7 +1324,7 @@ prefill_wide_kernel(uint16_t* __restrict__ out, const uint16_t* __restrict__ q, 
     float mx = fmaxf(fmaxf(fmaxf(part[0], part[1]), part[2]), fmaxf(fmaxf(part[3], part[4]), s[A][15]));
     float xa, xb;
     swap_rows(mx, true, xa, xb);
-    mx = max_of_numbers(xa, xb) * scale_log2;  // the scale is positive: the maximum commutes with it
+    mx = max_of_numbers(xa, xb) * scale_log2.k;  // the scale is positive: the maximum commutes with it
     const bool moves_up = mx > m + WIDE_RESCALE_SLACK;
     if (__any(moves_up)) {
       accumulate_values(vs + B * V_TILE, pp0, pp1);
@@ -1363,8 +1388,8 @@ prefill_wide_kernel(uint16_t* __restrict__ out, const uint16_t* __restrict__ q, 
       float sum0 = 0.f, sum1 = 0.f;
 #pragma unroll
       for (int e = 0; e < 16; e += 2) {
-        s[A][e] = fast_exp2(fmaf(s[A][e], scale_log2, -m_use));
-        s[A][e + 1] = fast_exp2(fmaf(s[A][e + 1], scale_log2, -m_use));
+        s[A][e] = fast_exp2(fmaf(s[A][e], scale_log2.k, -m_use));
+        s[A][e + 1] = fast_exp2(fmaf(s[A][e + 1], scale_log2.k, -m_use));
         sum0 += s[A][e];
         sum1 += s[A][e + 1];
       }
@@ -1521,7 +1546,7 @@ static int launch_prefill_wide(hipStream_t stream, uint16_t* out, const uint16_t
                                const uint16_t* k_pages, const uint16_t* v_pages, const int* block_table,
                                int table_width, const int* query_start_loc, const int* context_lens,
                                const int* blocks, int num_blocks, int heads, int kv_heads, int shift,
-                               float scale_log2, int window, int max_context, const int* ranges,
+                               ScoreRule scale_log2, int window, int max_context, const int* ranges,
                                float* partial_acc, float* partial_ml, const int* combine, int num_combine) {
   constexpr size_t lds = (size_t)2 * (K_TILE + V_TILE) * sizeof(uint16_t);
   static_assert(lds <= 64 * 1024, "two workgroups' staged windows must fit in LDS");
@@ -1598,7 +1623,7 @@ extern "C" int TS_SYM(ts_attention_decode_d)(
     void* out, void* partial_acc, void* partial_ml, const void* q, long q_stride, const void* k_pages,
     const void* v_pages, const int* block_table, int table_width, const int* query_start_loc,
     const int* context_lens, int seq_begin, int requests, int heads, int kv_heads, int block_size,
-    float scale, int window, int keys_per_split, int splits, const int* max_context, hipStream_t stream) {
+    float scale, float softcap, int window, int keys_per_split, int splits, const int* max_context, hipStream_t stream) {
   if (requests == 0) return TS_OK;
   if (!out || !partial_acc || !partial_ml || !q || !k_pages || !v_pages || !block_table ||
       !query_start_loc || !context_lens)
@@ -1617,7 +1642,7 @@ extern "C" int TS_SYM(ts_attention_decode_d)(
   hipLaunchKernelGGL(decode_kernel<DECODE_ONCE>, grid, dim3(64), 0, stream, (float*)partial_acc, (float*)partial_ml,
                      (const uint16_t*)q, q_stride, (const uint16_t*)k_pages, (const uint16_t*)v_pages,
                      block_table, table_width, query_start_loc, context_lens, seq_begin, heads, kv_heads,
-                     shift, scale * LOG2E, window, keys_per_split, splits, max_context);
+                     shift, score_rule(scale, softcap), window, keys_per_split, splits, max_context);
   if (hipGetLastError() != hipSuccess) return TS_ERR_LAUNCH;
   hipLaunchKernelGGL(decode_reduce_kernel, dim3(requests, heads), dim3(REDUCE_THREADS), 0, stream, (uint16_t*)out,
                      (const float*)partial_acc, (const float*)partial_ml, query_start_loc, seq_begin, heads,
@@ -1663,7 +1688,7 @@ extern "C" void TS_SYM(ts_attention_prefill_shape_d)(int heads, int kv_heads, in
 extern "C" int TS_SYM(ts_attention_prefill_d)(
     void* out, const void* q, long q_stride, const void* k_pages, const void* v_pages, const int* block_table,
     int table_width, const int* query_start_loc, const int* context_lens, const int* blocks, int num_blocks,
-    int block_rows, int heads, int kv_heads, int block_size, float scale, int window, int max_context,
+    int block_rows, int heads, int kv_heads, int block_size, float scale, float softcap, int window, int max_context,
     const int* ranges, void* partial_acc, void* partial_ml, const int* combine, int num_combine,
     hipStream_t stream) {
   if (num_blocks == 0) return TS_OK;
@@ -1681,7 +1706,7 @@ extern "C" int TS_SYM(ts_attention_prefill_d)(
   if (gsize >= 3)
     return launch_prefill_wide(stream, (uint16_t*)out, (const uint16_t*)q, q_stride, (const uint16_t*)k_pages,
                                (const uint16_t*)v_pages, block_table, table_width, query_start_loc, context_lens,
-                               blocks, num_blocks, heads, kv_heads, shift, scale * LOG2E, window, max_context, ranges,
+                               blocks, num_blocks, heads, kv_heads, shift, score_rule(scale, softcap), window, max_context, ranges,
                                (float*)partial_acc, (float*)partial_ml, combine, num_combine);
 #endif
   if (ranges) return TS_ERR_ARG;  // only blocks of 32 rows are shared out
@@ -1691,10 +1716,10 @@ extern "C" int TS_SYM(ts_attention_prefill_d)(
     if (gsize >= 5)
       return launch_prefill_shared<2>(stream, (uint16_t*)out, (const uint16_t*)q, q_stride, (const uint16_t*)k_pages,
                                          (const uint16_t*)v_pages, block_table, table_width, query_start_loc,
-                                         context_lens, blocks, num_blocks, heads, kv_heads, shift, scale * LOG2E, window);
+                                         context_lens, blocks, num_blocks, heads, kv_heads, shift, score_rule(scale, softcap), window);
     return launch_prefill_shared<1>(stream, (uint16_t*)out, (const uint16_t*)q, q_stride, (const uint16_t*)k_pages,
                                        (const uint16_t*)v_pages, block_table, table_width, query_start_loc,
-                                       context_lens, blocks, num_blocks, heads, kv_heads, shift, scale * LOG2E, window);
+                                       context_lens, blocks, num_blocks, heads, kv_heads, shift, score_rule(scale, softcap), window);
   }
   constexpr int CT = TS_PREFILL_HEADS;
   const int head_chunks = (gsize + CT - 1) / CT;
@@ -1702,6 +1727,6 @@ extern "C" int TS_SYM(ts_attention_prefill_d)(
   dim3 grid(num_blocks, kv_heads * head_chunks);
   hipLaunchKernelGGL(prefill_kernel<CT>, grid, dim3(64), 0, stream, (uint16_t*)out, (const uint16_t*)q, q_stride,
                      (const uint16_t*)k_pages, (const uint16_t*)v_pages, block_table, table_width,
-                     query_start_loc, context_lens, blocks, heads, kv_heads, shift, scale * LOG2E, window);
+                     query_start_loc, context_lens, blocks, heads, kv_heads, shift, score_rule(scale, softcap), window);
   return ts_launch_status();
 }

@@ -250,3 +250,163 @@ extern "C" int ts_moe_combine(float* out, const float* pair_out, const float* we
     return TS_ERR_DTYPE;
   return ts_launch_status();
 }
+
+// ---------------------------------------------------------------------------------------------
+// Many tokens (prompt portions), bfloat16: the pairs are grouped by expert and every expert's
+// rows go through the matrix cores in tiles, so an expert's matrices are read once per 64 rows
+// instead of once per pair.
+//
+// ts_moe_group: order[P] = the pairs sorted by expert (within an expert in no fixed order: every
+// row is computed alone, so the order changes nothing), tile_first[E + 1] = the running count of
+// row tiles of MOE_TILE_ROWS (tile_first[E]: all of them), row_first[E + 1] = the running count of
+// rows.  One block.
+//
+// ts_moe_grouped_rows: out[order[r], :] for every sorted row r, a block per (row tile, 128 output
+// columns), found from tile_first; blocks beyond the last tile leave at once, so the grid is the
+// upper bound P / MOE_TILE_ROWS + E.  A wavefront holds 32 rows x 64 columns of
+// v_mfma_f32_16x16x32_bf16 accumulators and reads both operands straight from memory, 16 bytes a
+// lane (A: 8 consecutive k of a gathered input row; B: 8 consecutive k of a weight row).  K must
+// be a multiple of 32.
+// ---------------------------------------------------------------------------------------------
+#define MOE_TILE_ROWS 64
+#define MOE_TILE_COLS 128
+
+__global__ void __launch_bounds__(1024)
+moe_group_kernel(int* __restrict__ order, int* __restrict__ tile_first, int* __restrict__ row_first,
+                 const int* __restrict__ taken, int pairs, int experts) {
+  __shared__ int count[MOE_MAX_EXPERTS];
+  __shared__ int cursor[MOE_MAX_EXPERTS];
+  for (int e = threadIdx.x; e < experts; e += blockDim.x) count[e] = 0;
+  __syncthreads();
+  for (int p = threadIdx.x; p < pairs; p += blockDim.x) {
+    const int e = taken[p];
+    if (e >= 0 && e < experts) atomicAdd(&count[e], 1);
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int rows = 0, tiles = 0;
+    for (int e = 0; e < experts; ++e) {
+      row_first[e] = rows;
+      tile_first[e] = tiles;
+      cursor[e] = rows;
+      rows += count[e];
+      tiles += (count[e] + MOE_TILE_ROWS - 1) / MOE_TILE_ROWS;
+    }
+    row_first[experts] = rows;
+    tile_first[experts] = tiles;
+  }
+  __syncthreads();
+  for (int p = threadIdx.x; p < pairs; p += blockDim.x) {
+    const int e = taken[p];
+    if (e >= 0 && e < experts) order[atomicAdd(&cursor[e], 1)] = p;
+  }
+}
+
+extern "C" int ts_moe_group(int* order, int* tile_first, int* row_first, const int* taken, int pairs, int experts,
+                            hipStream_t stream) {
+  if (!order || !tile_first || !row_first || !taken || pairs < 1) return TS_ERR_ARG;
+  if (experts < 1 || experts > MOE_MAX_EXPERTS) return TS_ERR_SHAPE;
+  hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(1024), 0, stream, order, tile_first, row_first, taken, pairs, experts);
+  return ts_launch_status();
+}
+
+typedef __bf16 moe_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float moe_f32x4 __attribute__((ext_vector_type(4)));
+
+template <bool GATED>
+__global__ void __launch_bounds__(256)
+moe_grouped_rows_kernel(void* __restrict__ out_any, const bf16_t* __restrict__ in, const bf16_t* __restrict__ weight,
+                        const int* __restrict__ order, const int* __restrict__ tile_first,
+                        const int* __restrict__ row_first, int in_share, int n, int k, int experts, GluRule rule) {
+  __shared__ int found[2];
+  const int tile = blockIdx.x;
+  if (tile >= tile_first[experts]) return;
+  if (threadIdx.x < TS_WAVE) {
+    // The expert whose tiles hold this one: the last e with tile_first[e] <= tile.
+    int best = -1;
+    for (int e = threadIdx.x; e < experts; e += TS_WAVE)
+      if (tile_first[e] <= tile && tile_first[e + 1] > tile) best = e;
+    best = (int)wave_max((float)best);
+    if (threadIdx.x == 0) found[0] = best;
+  }
+  __syncthreads();
+  const int e = found[0];
+  const int wave = threadIdx.x / TS_WAVE, lane = threadIdx.x % TS_WAVE;
+  const int r16 = lane % 16, group = lane / 16;
+  const int rows_begin = row_first[e] + (tile - tile_first[e]) * MOE_TILE_ROWS;
+  const int rows_end = row_first[e + 1];
+  const int row0 = rows_begin + (wave / 2) * 32;       // this wavefront's 32 sorted rows
+  const int col0 = blockIdx.y * MOE_TILE_COLS + (wave % 2) * 64;  // and its 64 columns
+  if (row0 >= rows_end || col0 >= n) return;
+  const bf16_t* w = weight + (size_t)e * n * k;
+  const bf16_t* a_row[2];
+  int pair_of[2];
+#pragma unroll
+  for (int a = 0; a < 2; ++a) {
+    const int r = min(row0 + 16 * a + r16, rows_end - 1);
+    pair_of[a] = order[r];
+    a_row[a] = in + (size_t)(pair_of[a] / in_share) * k + 8 * group;
+  }
+  const bf16_t* b_row[4];
+#pragma unroll
+  for (int b = 0; b < 4; ++b) b_row[b] = w + (size_t)min(col0 + 16 * b + r16, n - 1) * k + 8 * group;
+  moe_f32x4 acc[2][4];
+#pragma unroll
+  for (int a = 0; a < 2; ++a)
+#pragma unroll
+    for (int b = 0; b < 4; ++b) acc[a][b] = moe_f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int k0 = 0; k0 < k; k0 += 32) {
+    ts_u32x4 af[2], bf[4];
+#pragma unroll
+    for (int a = 0; a < 2; ++a) af[a] = *reinterpret_cast<const ts_u32x4*>(a_row[a] + k0);
+#pragma unroll
+    for (int b = 0; b < 4; ++b) bf[b] = *reinterpret_cast<const ts_u32x4*>(b_row[b] + k0);
+#pragma unroll
+    for (int a = 0; a < 2; ++a)
+#pragma unroll
+      for (int b = 0; b < 4; ++b)
+        acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(moe_bf16x8, af[a]),
+                                                            __builtin_bit_cast(moe_bf16x8, bf[b]), acc[a][b], 0, 0, 0);
+  }
+  // acc[a][b][i] is row 16 a + 4 group + i, column 16 b + r16 of the wavefront's tile.
+#pragma unroll
+  for (int a = 0; a < 2; ++a) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int r = row0 + 16 * a + 4 * group + i;
+      // The row's pair: held by the lane whose r16 is 4 group + i of the same a.
+      const int pair = __shfl(pair_of[a], 4 * group + i, 64);
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        const int col = col0 + 16 * b + r16;
+        const float v = acc[a][b][i];
+        if (GATED) {
+          const float other = __shfl_xor(v, 1, 64);  // columns alternate gate, up
+          if ((r16 & 1) == 0 && r < rows_end && col + 1 < n)
+            ((bf16_t*)out_any)[(size_t)pair * (n / 2) + col / 2] = from_float<bf16_t>(gated_unit(v, other, rule));
+        } else if (r < rows_end && col < n) {
+          ((float*)out_any)[(size_t)pair * n + col] = v;
+        }
+      }
+    }
+  }
+}
+
+extern "C" int ts_moe_grouped_rows(void* out, const void* in, const void* weight, const int* order,
+                                   const int* tile_first, const int* row_first, int pairs, int in_share, int n, int k,
+                                   int experts, int gated, float steepness, float limit, float up_shift,
+                                   hipStream_t stream) {
+  if (pairs == 0) return TS_OK;
+  if (!out || !in || !weight || !order || !tile_first || !row_first) return TS_ERR_ARG;
+  if (n < 1 || k < 32 || k % 32 != 0 || in_share < 1 || experts < 1 || experts > MOE_MAX_EXPERTS || (gated && (n & 1)))
+    return TS_ERR_SHAPE;
+  if (((uintptr_t)in | (uintptr_t)weight) % 16 != 0) return TS_ERR_ARG;
+  const GluRule rule = {steepness, limit, up_shift};
+  const dim3 grid(pairs / MOE_TILE_ROWS + experts + 1, (n + MOE_TILE_COLS - 1) / MOE_TILE_COLS), block(256);
+  if (grid.y > 65535) return TS_ERR_SHAPE;
+  if (gated)
+    hipLaunchKernelGGL(moe_grouped_rows_kernel<true>, grid, block, 0, stream, out, (const bf16_t*)in, (const bf16_t*)weight, order, tile_first, row_first, in_share, n, k, experts, rule);
+  else
+    hipLaunchKernelGGL(moe_grouped_rows_kernel<false>, grid, block, 0, stream, out, (const bf16_t*)in, (const bf16_t*)weight, order, tile_first, row_first, in_share, n, k, experts, rule);
+  return ts_launch_status();
+}

@@ -62,6 +62,9 @@ _SIGNATURES: dict[str, dict[str, list]] = {
                          c_int, c_float, c_int, c_void_p],
         "ts_moe_pair_rows": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float,
                              c_float, c_float, c_int, c_void_p],
+        "ts_moe_group": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
+        "ts_moe_grouped_rows": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
+                                c_int, c_float, c_float, c_float, c_void_p],
         "ts_moe_combine": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_void_p, c_int, c_int, c_int,
                            c_int, c_void_p],
         "ts_gemm_plain": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_long, c_long,
@@ -84,10 +87,10 @@ def _attention_signatures(head_dim: int) -> dict[str, list]:
     return {
         f"ts_attention_decode_d{head_dim}": [c_void_p, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_void_p,
                                              c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
-                                             c_int, c_float, c_int, c_int, c_int, c_void_p, c_void_p],
+                                             c_int, c_float, c_float, c_int, c_int, c_int, c_void_p, c_void_p],
         f"ts_attention_prefill_d{head_dim}": [c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int,
                                               c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float,
-                                              c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p],
+                                              c_float, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p],
         f"ts_attention_prefill_rows_d{head_dim}": [c_int, c_int],
         f"ts_attention_prefill_shape_d{head_dim}": [c_int, c_int, c_int, c_void_p, c_void_p],
     }
@@ -655,14 +658,63 @@ class Ops:
                                           dtype_code(rows.dtype), self.stream()), "ts_moe_pair_rows")
         return out
 
+    #: From this many tokens on, a bfloat16 step's pairs are grouped by expert and go through the
+    #: matrix cores (below it every pair streams its expert's matrices, which is what few tokens cost anyway).
+    moe_grouped_min_tokens = 33
+
+    def moe_grouping(self, taken: torch.Tensor, experts: int, dtype: torch.dtype, *widths: int):
+        """``(order, tile_first, row_first)`` for :meth:`moe_grouped_rows` where a step's pairs are
+        worth grouping by expert (bfloat16, many tokens, every inner width a multiple of 32), else
+        ``None``.  All on the device: the host never sees who took which expert."""
+        _gpu(taken)
+        _i32(taken, "taken")
+        if (dtype != torch.bfloat16 or taken.shape[0] < self.moe_grouped_min_tokens or experts > 1024
+                or any(w % 32 != 0 for w in widths)):
+            return None
+        pairs = taken.numel()
+        order = torch.empty((pairs,), dtype=torch.int32, device=taken.device)
+        tile_first = torch.empty((experts + 1,), dtype=torch.int32, device=taken.device)
+        row_first = torch.empty((experts + 1,), dtype=torch.int32, device=taken.device)
+        _check(self.core.ts_moe_group(_ptr(order), _ptr(tile_first), _ptr(row_first), _ptr(taken), pairs, experts,
+                                      self.stream()), "ts_moe_group")
+        return order, tile_first, row_first
+
+    def moe_grouped_rows(self, rows: torch.Tensor, weight: torch.Tensor, grouping: tuple, pairs: int, *, share: int,
+                         rule: tuple[float, float, float] | None = None) -> torch.Tensor:
+        """What :meth:`moe_pair_rows` computes, for bfloat16 pairs grouped by expert
+        (:meth:`moe_grouping`), on the matrix cores."""
+        _gpu(rows, weight)
+        order, tile_first, row_first = grouping
+        _need(weight.dim() == 3 and weight.is_contiguous() and rows.dim() == 2 and rows.is_contiguous()
+              and rows.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and rows.shape[1] == weight.shape[2],
+              "rows [*, K] and weight [E, N, K] must be bfloat16")
+        experts, n, k = weight.shape
+        _need(k % 32 == 0 and share >= 1 and rows.shape[0] * share >= pairs and order.numel() == pairs
+              and tile_first.numel() == experts + 1, "grouping and sizes do not fit")
+        if rule is not None:
+            _need(n % 2 == 0, "a gated stack has an even number of rows")
+            out = torch.empty((pairs, n // 2), dtype=torch.bfloat16, device=rows.device)
+        else:
+            out = torch.empty((pairs, n), dtype=torch.float32, device=rows.device)
+        r = rule or (1.0, 0.0, 0.0)
+        _check(self.core.ts_moe_grouped_rows(_ptr(out), _ptr(rows), _ptr(weight), _ptr(order), _ptr(tile_first),
+                                             _ptr(row_first), pairs, share, n, k, experts, 0 if rule is None else 1,
+                                             float(r[0]), float(r[1]), float(r[2]), self.stream()), "ts_moe_grouped_rows")
+        return out
+
     def moe_expert_units(self, x: torch.Tensor, gate_up: torch.Tensor, taken: torch.Tensor,
-                         rule: tuple[float, float, float]) -> torch.Tensor:
+                         rule: tuple[float, float, float], grouping: tuple | None = None) -> torch.Tensor:
         """The gated units ``[T * top, I]`` of every (token, taken expert) pair: ``x [T, H]`` against
         the pair's expert's matrix of the stack ``gate_up [E, 2 I, H]`` (rows alternate gate, up)."""
+        if grouping is not None:
+            return self.moe_grouped_rows(x, gate_up, grouping, taken.numel(), share=taken.shape[1], rule=rule)
         return self.moe_pair_rows(x, gate_up, taken, share=taken.shape[1], rule=rule)
 
-    def moe_expert_outputs(self, units: torch.Tensor, down: torch.Tensor, taken: torch.Tensor) -> torch.Tensor:
+    def moe_expert_outputs(self, units: torch.Tensor, down: torch.Tensor, taken: torch.Tensor,
+                           grouping: tuple | None = None) -> torch.Tensor:
         """``[T * top, H]`` float32: every pair's units against its expert's matrix of ``down [E, H, I]``."""
+        if grouping is not None:
+            return self.moe_grouped_rows(units, down, grouping, taken.numel(), share=1)
         return self.moe_pair_rows(units, down, taken, share=1)
 
     def moe_combine(self, pair_out: torch.Tensor, weights: torch.Tensor, extra: torch.Tensor | None = None,
@@ -741,12 +793,11 @@ class Ops:
         return out
 
     @staticmethod
-    def mfma_attention_supported(dtype: torch.dtype, head_dim: int, block_size: int, softcap: float = 0.0) -> bool:
+    def mfma_attention_supported(dtype: torch.dtype, head_dim: int, block_size: int) -> bool:
         """Whether the matrix-core attention kernels take this geometry (bfloat16, head sizes
-        16..256 in steps of 16, pages of at least 8 tokens, no cap on the scores); anything else
-        runs the generic kernel."""
-        return (dtype == torch.bfloat16 and head_dim % 16 == 0 and 16 <= head_dim <= 256 and block_size >= 8
-                and not softcap)
+        16..256 in steps of 16, pages of at least 8 tokens); anything else runs the generic
+        kernel."""
+        return dtype == torch.bfloat16 and head_dim % 16 == 0 and 16 <= head_dim <= 256 and block_size >= 8
 
     def attention_decode(
         self,
@@ -765,6 +816,7 @@ class Ops:
         window: int | None,
         max_context: int,
         max_context_dev: torch.Tensor | None = None,
+        softcap: float = 0.0,
     ) -> None:
         """Matrix-core attention for the single-token requests ``seq_begin .. seq_begin +
         requests - 1`` of the step; writes their rows of ``out [T, heads * D]``.  ``max_context``
@@ -799,7 +851,7 @@ class Ops:
         fn = getattr(lib, f"ts_attention_decode_d{head_dim}")
         _check(fn(_ptr(out), _ptr(partial_acc), _ptr(partial_ml), _ptr(q), q_stride, _ptr(k_pages), _ptr(v_pages),
                   _ptr(block_table), block_table.shape[1], _ptr(query_start_loc), _ptr(context_lens), seq_begin,
-                  requests, heads, kv_heads, block_size, float(scale), int(window or 0), keys_per_split, splits,
+                  requests, heads, kv_heads, block_size, float(scale), float(softcap), int(window or 0), keys_per_split, splits,
                   _ptr(max_context_dev), self.stream()), "ts_attention_decode")
 
     def prefill_block_rows(self, head_dim: int, heads: int, kv_heads: int) -> int:
@@ -856,6 +908,7 @@ class Ops:
         window: int | None,
         max_context: int,
         block_rows: int = 16,
+        softcap: float = 0.0,
     ) -> None:
         """Matrix-core attention for blocks of ``block_rows`` consecutive rows of multi-token
         requests (what :meth:`prefill_block_rows` says for the geometry): ``blocks`` is the work
@@ -895,7 +948,7 @@ class Ops:
         fn = getattr(lib, f"ts_attention_prefill_d{head_dim}")
         _check(fn(_ptr(out), _ptr(q), q_stride, _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
                   block_table.shape[1], _ptr(query_start_loc), _ptr(context_lens), _ptr(blocks), blocks.shape[0],
-                  block_rows, heads, kv_heads, block_size, float(scale), int(window or 0), int(max_context),
+                  block_rows, heads, kv_heads, block_size, float(scale), float(softcap), int(window or 0), int(max_context),
                   _ptr(work.ranges), _ptr(partial_acc), _ptr(partial_ml), _ptr(work.combine), num_combine,
                   self.stream()),
                "ts_attention_prefill")

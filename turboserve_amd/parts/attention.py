@@ -167,9 +167,9 @@ class GroupedQueryAttention(Mixer):
         table = ctx.block_tables[cache.group]
         slopes = self.position.score_slopes(self.num_heads)
         fast = (slopes is None and self.value_dim == self.head_dim
-                and ops.mfma_attention_supported(qkv.dtype, self.head_dim, cache.block_size, self.softcap))
+                and ops.mfma_attention_supported(qkv.dtype, self.head_dim, cache.block_size))
         if fast:
-            out = ops.rows_buffer(ctx.num_tokens, self.q_size, qkv.dtype, qkv.device)
+            out = ops.rows_buffer(ctx.num_tokens, self.out_size, qkv.dtype, qkv.device)
             if ctx.num_prefill_seqs > 0:
                 # The launch's list of row blocks is the same for every layer with this geometry.
                 rows = ops.prefill_block_rows(self.head_dim, self.num_heads, self.num_kv_heads)
@@ -180,13 +180,14 @@ class GroupedQueryAttention(Mixer):
                 ops.attention_prefill(
                     out, qkv, q_stride, cache.k, cache.v, table, ctx.query_start_loc, ctx.context_lens,
                     blocks, self.num_heads, self.scale, self.window, ctx.max_prefill_context_len, rows,
+                    softcap=self.softcap,
                 )
             if ctx.num_decode_seqs > 0:
                 ops.attention_decode(
                     out, qkv, q_stride, cache.k, cache.v, table, ctx.query_start_loc, ctx.context_lens,
                     ctx.num_prefill_seqs, ctx.num_decode_seqs, self.num_heads, self.scale, self.window,
                     min(ctx.max_decode_context_len, table.shape[1] * cache.block_size),
-                    ctx.max_decode_context_dev,
+                    ctx.max_decode_context_dev, softcap=self.softcap,
                 )
             return out
         return ops.paged_attention_generic(

@@ -26,8 +26,9 @@ class RoutedExperts(FeedForward):
 
     The experts' matrices are stacked at load: ``[E, 2 I, H]`` with rows alternating gate, up,
     and ``[E, H, I]``.  A step routes on the device, runs every (token, taken expert) pair
-    against its expert's matrices and sums with the weights, so nothing depends on data the
-    host has not seen and single-token steps can be recorded.
+    against its expert's matrices (pair by pair in steps of few tokens, grouped by expert on the
+    matrix cores in bfloat16 steps of many) and sums with the weights, so nothing depends on data
+    the host has not seen and single-token steps can be recorded.
     """
 
     def __init__(
@@ -119,7 +120,8 @@ class RoutedExperts(FeedForward):
         ops = self.runtime.ops
         taken, weights, gate = ops.moe_route(x, self.router, top=self.top, groups=self.groups, keep=self.keep,
                                              scale=self.route_scale, extra=self.shared_gate)
-        units = ops.moe_expert_units(x, self.gate_up, taken, self.rule)
-        outputs = ops.moe_expert_outputs(units, self.down, taken)
+        grouping = ops.moe_grouping(taken, self.experts, x.dtype, self.hidden_size, self.expert_size)
+        units = ops.moe_expert_units(x, self.gate_up, taken, self.rule, grouping)
+        outputs = ops.moe_expert_outputs(units, self.down, taken, grouping)
         extra = self.shared.forward(x, ctx) if self.shared is not None else None
         return ops.moe_combine(outputs, weights, extra, gate, x.dtype)
