@@ -498,9 +498,10 @@ def design_pair(size: str) -> tuple[dict, dict]:
     return sisisun, qwen2
 
 
-def active_weight_elements(model, batch: int) -> float:
+def active_weight_elements(model, batch: int, *, per_token: bool = False) -> float:
     """Elements of the weights a step of ``batch`` tokens reads: every tensor of every layer run
-    once, but of a routed feed-forward's experts only as many as ``batch`` tokens can take."""
+    once, but of a routed feed-forward's experts only as many as ``batch`` tokens can take.  With
+    ``per_token``: the elements one token is multiplied with (of the experts: those it takes)."""
     from turboserve_amd.parts.experts import RoutedExperts
 
     total = 0.0
@@ -512,7 +513,7 @@ def active_weight_elements(model, batch: int) -> float:
             for dim in spec.shape:
                 count *= dim
             if isinstance(forward, RoutedExperts) and name.startswith(forward._expert(0, 1).rsplit("e0", 1)[0] + "e"):
-                count *= min(1.0, batch * forward.top / forward.experts)
+                count *= forward.top / forward.experts if per_token else min(1.0, batch * forward.top / forward.experts)
             total += count
     head = model.plan.vocab_size * model.plan.hidden_size
     return total + head
@@ -533,18 +534,22 @@ def run_designs(sizes: list[str], dtype_name: str, steps: int, warmup: int) -> d
     batch, context, prompt = 8, 2048, 2048
     out: dict = {"dtype": dtype_name, "decode": f"{batch} requests at {context} tokens", "prefill": f"{prompt} tokens"}
     for size in sizes:
+        size, _, only = size.partition(":")  # "2k:qwen2": that design alone; "2k:qwen2:prefill": that phase alone (for profiles)
+        only, _, phase = only.partition(":")
         for label, shape in zip(("sisisun", "qwen2"), design_pair(size)):
+            if only and only != label:
+                continue
             runtime = make_runtime(dtype, "cuda:0")
             config, model = build_model(shape, runtime)
             random_tensors_on_device(model, seed=0)
-            seconds = run_prefill(model, config, prompt, tune=False)
-            decode = run_decode(model, config, batch, context - 1, steps=steps, warmup=warmup)
+            decode = run_decode(model, config, batch, context - 1, steps=steps, warmup=warmup) if phase != "prefill" \
+                else {"mean_context": context, "step_seconds": float("inf"), "tokens_per_s": 0.0}
+            seconds = run_prefill(model, config, prompt, tune=False) if phase != "decode" else float("inf")
             needs = [need for need in model.cache_needs() if need is not None]
             kv_elements = sum(n.num_kv_heads * (n.head_dim + n.value_width) for n in needs)
             read = (active_weight_elements(model, batch) + batch * decode["mean_context"] * kv_elements) * itemsize
-            attention = sum(4.0 * prompt * prompt / 2 * (n.head_dim + n.value_width) / 2 for n in needs)  # causal
             heads_per_kv = [model.blocks[c.layer].mixer.num_heads // model.blocks[c.layer].mixer.num_kv_heads for c in model.plan.schedule]
-            flops = 2.0 * prompt * (active_weight_elements(model, prompt) - model.plan.vocab_size * model.plan.hidden_size) \
+            flops = 2.0 * prompt * (active_weight_elements(model, prompt, per_token=True) - model.plan.vocab_size * model.plan.hidden_size) \
                 + sum(4.0 * prompt * prompt / 2 * n.num_kv_heads * g * (n.head_dim + n.value_width) / 2 for n, g in zip(needs, heads_per_kv))
             out[f"{size}_{label}"] = {
                 "layer_runs": len(model.plan.schedule), "parameters_M": round(model.num_parameters() / 1e6, 1),

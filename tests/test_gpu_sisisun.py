@@ -123,8 +123,10 @@ def test_the_router_takes_what_the_rule_says(ops, experts, top, groups, keep):
     x = torch.randn(tokens, hidden, generator=g)
     router = torch.randn(experts, hidden, generator=g) * 0.4
     extra = torch.randn(hidden, generator=g) * 0.3
-    taken, weights, gate = ops.moe_route(x.to(DEV), router.to(DEV), top=top, groups=groups, keep=keep, scale=1.7,
-                                         extra=extra.to(DEV))
+    with_gate = torch.cat([router, extra.view(1, -1)], dim=0)
+    taken, weights, gate = ops.moe_route(x.to(DEV), with_gate.to(DEV), top=top, groups=groups, keep=keep, scale=1.7,
+                                         experts=experts)
+    assert ops.moe_route(x.to(DEV), router.to(DEV), top=top, groups=groups, keep=keep, scale=1.7)[2] is None
     scores = torch.sigmoid(x @ router.T)
     for t in range(tokens):
         want = plain.route(scores[t].tolist(), top, groups, keep)

@@ -17,8 +17,16 @@
 
 template <typename P>
 __device__ __forceinline__ float sum_of_splits(const P* p, int splits, size_t stride) {
-  float s = to_float(p[0]);
-  for (int i = 1; i < splits; ++i) s += to_float(p[(size_t)i * stride]);
+  if (splits == 1) return to_float(p[0]);
+  float s = 0.f;
+  for (int first = 0; first < splits; first += 8) {  // eight loads in flight, added in split order
+    float v[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = to_float(p[(size_t)min(first + j, splits - 1) * stride]);
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      if (first + j < splits) s += v[j];
+  }
   return s;
 }
 
@@ -135,6 +143,26 @@ value_store_kernel(const P* proj, int splits, size_t split_stride, T* __restrict
   }
 }
 
+// Values of few tokens, or of partial sums: a thread per (token, value dimension), so that the
+// loads of a step of single tokens are all in flight at once.
+template <typename T, typename P>
+__global__ void __launch_bounds__(256)
+value_store_few_kernel(const P* proj, int splits, size_t split_stride, T* __restrict__ v_pages,
+                       const int* __restrict__ slots, int tokens, int heads, int kv_heads, int dim, int vdim,
+                       int block_size) {
+  const int t = blockIdx.x;
+  const int slot = slots[t];
+  if (slot < 0) return;
+  const size_t width = (size_t)(heads + kv_heads) * dim + (size_t)kv_heads * vdim;
+  const P* values = proj + (size_t)t * width + (size_t)(heads + kv_heads) * dim;
+  const size_t page = (size_t)(slot / block_size) * kv_heads;
+  const int offset = slot % block_size;
+  for (int i = threadIdx.x; i < kv_heads * vdim; i += blockDim.x) {
+    const int kvh = i / vdim, d = i % vdim;
+    v_pages[((page + kvh) * vdim + d) * block_size + offset] = from_float<T>(sum_of_splits(values + i, splits, split_stride));
+  }
+}
+
 template <typename T, typename P>
 static void launch_head_norm_store(void* q_out, long q_stride, const void* proj, int splits, long split_stride,
                                    void* k_pages, void* v_pages, const void* q_gain, const void* k_gain, float eps,
@@ -146,7 +174,10 @@ static void launch_head_norm_store(void* q_out, long q_stride, const void* proj,
                      dim3(64 * HNS_WAVES), 0, stream, (T*)q_out, q_stride, (const P*)proj, splits, (size_t)split_stride,
                      (T*)k_pages, (const T*)q_gain, (const T*)k_gain, eps, gain_offset, cos_table, sin_table, positions,
                      slots, tokens, heads, kv_heads, dim, vdim, block_size);
-  if (slots)
+  if (slots && (tokens < 4 * HNS_GROUP || splits > 1))
+    hipLaunchKernelGGL((value_store_few_kernel<T, P>), dim3(tokens), dim3(256), 0, stream, (const P*)proj, splits,
+                       (size_t)split_stride, (T*)v_pages, slots, tokens, heads, kv_heads, dim, vdim, block_size);
+  else if (slots)
     hipLaunchKernelGGL((value_store_kernel<T, P>), dim3((tokens + HNS_GROUP - 1) / HNS_GROUP, kv_heads), dim3(64), 0,
                        stream, (const P*)proj, splits, (size_t)split_stride, (T*)v_pages, slots, tokens, heads, kv_heads,
                        dim, vdim, block_size);

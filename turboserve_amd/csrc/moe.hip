@@ -1,7 +1,8 @@
 // Routed feed-forward ("mixture of experts"): the router with its selection rule, the experts'
 // products for the (token, taken expert) pairs of a step, and the weighted sum.
 //
-// Router, all in 32-bit: z = R x, s = sigmoid(z).  The experts form `groups` equal groups of
+// Router: z = R x comes from the engine's own product with a 32-bit result; here, all in 32-bit,
+// s = sigmoid(z).  The experts form `groups` equal groups of
 // neighbours; a group's mark is the sum of its two largest s (its one s if it has one member);
 // only experts of the `keep` groups with the largest marks can be taken; the `top` of them with
 // the largest s are, with weights s / (sum of the taken s + 1e-20) * route_scale.  Equal values go
@@ -11,13 +12,6 @@
 #define MOE_MAX_EXPERTS 1024
 #define MOE_MAX_TOP 32
 
-template <typename T>
-__device__ __forceinline__ float lanes_dot(const T* __restrict__ a, const T* __restrict__ b, int n, int lane) {
-  float s = 0.f;
-  for (int k = lane; k < n; k += TS_WAVE) s = fmaf(to_float(a[k]), to_float(b[k]), s);
-  return wave_sum(s);
-}
-
 // Index of the largest of the values the lanes hold (value, index pairs; index < 2^24), the
 // lower index among equals; every lane returns it.  A lane without a candidate passes -inf.
 __device__ __forceinline__ int wave_argmax(float value, int index, float& best) {
@@ -26,31 +20,24 @@ __device__ __forceinline__ int wave_argmax(float value, int index, float& best) 
   return (int)(-wave_max(mine));
 }
 
-// One block of 256 threads per token.
-template <typename T>
-__global__ void __launch_bounds__(256)
-moe_route_kernel(int* __restrict__ taken, float* __restrict__ weights, float* __restrict__ extra_gate,
-                 const T* __restrict__ x, const T* __restrict__ router, const T* __restrict__ extra, int width,
-                 int experts, int top, int groups, int keep, float route_scale) {
+// One wavefront per token: the selection from the router's 32-bit outputs z [T, stride] (the
+// first `experts` of a row; where extra_gate is asked for, element `experts` of the row is the
+// gate's own output).
+__global__ void __launch_bounds__(TS_WAVE)
+moe_select_kernel(int* __restrict__ taken, float* __restrict__ weights, float* __restrict__ extra_gate,
+                  const float* __restrict__ z, int stride, int experts, int top, int groups, int keep,
+                  float route_scale) {
   __shared__ float score[MOE_MAX_EXPERTS];
   __shared__ float mark[MOE_MAX_EXPERTS];   // per group
   __shared__ int open_group[MOE_MAX_EXPERTS];
   const int t = blockIdx.x;
-  const int wave = threadIdx.x / TS_WAVE, lane = threadIdx.x % TS_WAVE, waves = blockDim.x / TS_WAVE;
-  const T* row = x + (size_t)t * width;
-  for (int e = wave; e < experts; e += waves) {
-    const float z = lanes_dot(router + (size_t)e * width, row, width, lane);
-    if (lane == 0) score[e] = 1.f / (1.f + expf(-z));
-  }
-  if (extra_gate && wave == waves - 1) {
-    const float z = lanes_dot(extra, row, width, lane);
-    if (lane == 0) extra_gate[t] = 1.f / (1.f + expf(-z));
-  }
+  const int lane = threadIdx.x;
+  const float* row = z + (size_t)t * stride;
+  for (int e = lane; e < experts; e += TS_WAVE) score[e] = 1.f / (1.f + expf(-row[e]));
+  if (extra_gate && lane == 0) extra_gate[t] = 1.f / (1.f + expf(-row[experts]));
   __syncthreads();
-  // The selection is the first wavefront's; the others only keep the barriers company.
-  const bool lead = wave == 0;
   const int size = experts / groups;
-  if (lead) {
+  {
     for (int g = lane; g < groups; g += TS_WAVE) {
       float a = -INFINITY, b = -INFINITY;  // largest, second
       for (int i = 0; i < size; ++i) {
@@ -64,7 +51,7 @@ moe_route_kernel(int* __restrict__ taken, float* __restrict__ weights, float* __
   __syncthreads();
   if (keep < groups) {
     for (int round = 0; round < keep; ++round) {
-      if (lead) {
+      {
         float mine = -INFINITY;
         int at = 0;
         for (int g = lane; g < groups; g += TS_WAVE)
@@ -80,7 +67,7 @@ moe_route_kernel(int* __restrict__ taken, float* __restrict__ weights, float* __
   float kept_score = 0.f;  // lane r holds the score of the r-th taken expert
   int kept_index = 0;
   for (int round = 0; round < top; ++round) {
-    if (lead) {
+    {
       float mine = -INFINITY;
       int at = 0;
       for (int e = lane; e < experts; e += TS_WAVE)
@@ -93,26 +80,21 @@ moe_route_kernel(int* __restrict__ taken, float* __restrict__ weights, float* __
     }
     __syncthreads();
   }
-  if (lead && lane < top) {
+  if (lane < top) {
     taken[(size_t)t * top + lane] = kept_index;
     weights[(size_t)t * top + lane] = kept_score / (total + 1e-20f) * route_scale;
   }
 }
 
-extern "C" int ts_moe_route(int* taken, float* weights, float* extra_gate, const void* x, const void* router,
-                            const void* extra, int tokens, int width, int experts, int top, int groups, int keep,
-                            float route_scale, int dtype, hipStream_t stream) {
+extern "C" int ts_moe_select(int* taken, float* weights, float* extra_gate, const float* z, int tokens, int stride,
+                             int experts, int top, int groups, int keep, float route_scale, hipStream_t stream) {
   if (tokens == 0) return TS_OK;
-  if (!taken || !weights || !x || !router || (extra_gate && !extra)) return TS_ERR_ARG;
+  if (!taken || !weights || !z) return TS_ERR_ARG;
   if (experts < 1 || experts > MOE_MAX_EXPERTS || top < 1 || top > MOE_MAX_TOP || groups < 1 || experts % groups != 0 ||
-      keep < 1 || keep > groups || top > (experts / groups) * keep || width < 1)
+      keep < 1 || keep > groups || top > (experts / groups) * keep || stride < experts + (extra_gate ? 1 : 0))
     return TS_ERR_SHAPE;
-  if (dtype == TS_F32)
-    hipLaunchKernelGGL(moe_route_kernel<float>, dim3(tokens), dim3(256), 0, stream, taken, weights, extra_gate, (const float*)x, (const float*)router, (const float*)extra, width, experts, top, groups, keep, route_scale);
-  else if (dtype == TS_BF16)
-    hipLaunchKernelGGL(moe_route_kernel<bf16_t>, dim3(tokens), dim3(256), 0, stream, taken, weights, extra_gate, (const bf16_t*)x, (const bf16_t*)router, (const bf16_t*)extra, width, experts, top, groups, keep, route_scale);
-  else
-    return TS_ERR_DTYPE;
+  hipLaunchKernelGGL(moe_select_kernel, dim3(tokens), dim3(TS_WAVE), 0, stream, taken, weights, extra_gate, z, stride,
+                     experts, top, groups, keep, route_scale);
   return ts_launch_status();
 }
 
@@ -223,17 +205,17 @@ __global__ void moe_combine_kernel(float* __restrict__ out, const float* __restr
                                    const float* __restrict__ weights, const P* __restrict__ extra, int splits,
                                    size_t split_stride, const float* __restrict__ extra_gate, int top, int width) {
   const int t = blockIdx.x;
-  for (int i = threadIdx.x; i < width; i += blockDim.x) {
-    float s = 0.f;
-    for (int j = 0; j < top; ++j)
-      s = fmaf(weights[(size_t)t * top + j], pair_out[((size_t)t * top + j) * width + i], s);
-    if (extra) {
-      float x = 0.f;
-      for (int sp = 0; sp < splits; ++sp) x += to_float(extra[(size_t)sp * split_stride + (size_t)t * width + i]);
-      s = fmaf(extra_gate ? extra_gate[t] : 1.f, x, s);
-    }
-    out[(size_t)t * width + i] = s;
+  const int i = blockIdx.y * blockDim.x + threadIdx.x;
+  if (i >= width) return;
+  float s = 0.f;
+  for (int j = 0; j < top; ++j)
+    s = fmaf(weights[(size_t)t * top + j], pair_out[((size_t)t * top + j) * width + i], s);
+  if (extra) {
+    float x = 0.f;
+    for (int sp = 0; sp < splits; ++sp) x += to_float(extra[(size_t)sp * split_stride + (size_t)t * width + i]);
+    s = fmaf(extra_gate ? extra_gate[t] : 1.f, x, s);
   }
+  out[(size_t)t * width + i] = s;
 }
 
 extern "C" int ts_moe_combine(float* out, const float* pair_out, const float* weights, const void* extra,
@@ -241,7 +223,8 @@ extern "C" int ts_moe_combine(float* out, const float* pair_out, const float* we
                               int top, int width, int dtype, hipStream_t stream) {
   if (tokens == 0) return TS_OK;
   if (!out || !pair_out || !weights || top < 1 || width < 1 || splits < 1) return TS_ERR_ARG;
-  const dim3 grid(tokens), block(256);
+  const dim3 grid(tokens, (width + 255) / 256), block(256);
+  if (grid.y > 65535) return TS_ERR_SHAPE;
   if (!extra || extra_f32 || dtype == TS_F32)
     hipLaunchKernelGGL(moe_combine_kernel<float>, grid, block, 0, stream, out, pair_out, weights, (const float*)extra, splits, (size_t)split_stride, extra_gate, top, width);
   else if (dtype == TS_BF16)
@@ -263,10 +246,7 @@ extern "C" int ts_moe_combine(float* out, const float* pair_out, const float* we
 //
 // ts_moe_grouped_rows: out[order[r], :] for every sorted row r, a block per (row tile, 128 output
 // columns), found from tile_first; blocks beyond the last tile leave at once, so the grid is the
-// upper bound P / MOE_TILE_ROWS + E.  A wavefront holds 32 rows x 64 columns of
-// v_mfma_f32_16x16x32_bf16 accumulators and reads both operands straight from memory, 16 bytes a
-// lane (A: 8 consecutive k of a gathered input row; B: 8 consecutive k of a weight row).  K must
-// be a multiple of 32.
+// upper bound P / MOE_TILE_ROWS + E.  K must be a multiple of 8.
 // ---------------------------------------------------------------------------------------------
 #define MOE_TILE_ROWS 64
 #define MOE_TILE_COLS 128
@@ -313,72 +293,116 @@ extern "C" int ts_moe_group(int* order, int* tile_first, int* row_first, const i
 typedef __bf16 moe_bf16x8 __attribute__((ext_vector_type(8)));
 typedef float moe_f32x4 __attribute__((ext_vector_type(4)));
 
+#define MOE_DEPTH 64                   // k per iteration
+#define MOE_LDS_ROW (MOE_DEPTH + 8)    // elements; 144 bytes: sixteen rows' same piece lies in sixteen different banks' quads
+
+// A block of four wavefronts owns 64 sorted rows x 128 columns; per iteration both operands go
+// global memory -> registers (16-byte pieces, eight consecutive threads a row's 128 bytes) -> LDS ->
+// matrix cores, and the loads of the next iteration are in flight while this one's products run.
+// A wavefront computes 32 rows x 64 columns (2 x 4 tiles of 16 x 16).
 template <bool GATED>
 __global__ void __launch_bounds__(256)
 moe_grouped_rows_kernel(void* __restrict__ out_any, const bf16_t* __restrict__ in, const bf16_t* __restrict__ weight,
                         const int* __restrict__ order, const int* __restrict__ tile_first,
                         const int* __restrict__ row_first, int in_share, int n, int k, int experts, GluRule rule) {
-  __shared__ int found[2];
+  __shared__ __attribute__((aligned(16))) uint16_t a_tile[MOE_TILE_ROWS * MOE_LDS_ROW];
+  __shared__ __attribute__((aligned(16))) uint16_t b_tile[MOE_TILE_COLS * MOE_LDS_ROW];
+  __shared__ int found;
   const int tile = blockIdx.x;
-  if (tile >= tile_first[experts]) return;
+  if (tile >= tile_first[experts]) return;  // the whole block leaves together
   if (threadIdx.x < TS_WAVE) {
-    // The expert whose tiles hold this one: the last e with tile_first[e] <= tile.
+    // The expert whose tiles hold this one.
     int best = -1;
     for (int e = threadIdx.x; e < experts; e += TS_WAVE)
       if (tile_first[e] <= tile && tile_first[e + 1] > tile) best = e;
     best = (int)wave_max((float)best);
-    if (threadIdx.x == 0) found[0] = best;
+    if (threadIdx.x == 0) found = best;
   }
   __syncthreads();
-  const int e = found[0];
-  const int wave = threadIdx.x / TS_WAVE, lane = threadIdx.x % TS_WAVE;
+  const int e = found;
+  const int tid = threadIdx.x;
+  const int wave = tid / TS_WAVE, lane = tid % TS_WAVE;
   const int r16 = lane % 16, group = lane / 16;
+  const int wm = wave / 2, wn = wave % 2;
   const int rows_begin = row_first[e] + (tile - tile_first[e]) * MOE_TILE_ROWS;
   const int rows_end = row_first[e + 1];
-  const int row0 = rows_begin + (wave / 2) * 32;       // this wavefront's 32 sorted rows
-  const int col0 = blockIdx.y * MOE_TILE_COLS + (wave % 2) * 64;  // and its 64 columns
-  if (row0 >= rows_end || col0 >= n) return;
+  const int col_begin = blockIdx.y * MOE_TILE_COLS;
   const bf16_t* w = weight + (size_t)e * n * k;
-  const bf16_t* a_row[2];
-  int pair_of[2];
+
+  // What this thread fetches per iteration: pieces tid + 256 i of the tiles, piece = (row, 8 k).
+  const int piece_k = 8 * (tid % 8);
+  const int piece_row = tid / 8;  // + 32 i
+  const bf16_t* a_src[2];
+  const bf16_t* b_src[4];
 #pragma unroll
-  for (int a = 0; a < 2; ++a) {
-    const int r = min(row0 + 16 * a + r16, rows_end - 1);
-    pair_of[a] = order[r];
-    a_row[a] = in + (size_t)(pair_of[a] / in_share) * k + 8 * group;
+  for (int i = 0; i < 2; ++i) {
+    const int r = min(rows_begin + piece_row + 32 * i, rows_end - 1);
+    a_src[i] = in + (size_t)(order[r] / in_share) * k;
   }
-  const bf16_t* b_row[4];
 #pragma unroll
-  for (int b = 0; b < 4; ++b) b_row[b] = w + (size_t)min(col0 + 16 * b + r16, n - 1) * k + 8 * group;
+  for (int i = 0; i < 4; ++i) b_src[i] = w + (size_t)min(col_begin + piece_row + 32 * i, n - 1) * k;
+  ts_u32x4 a_reg[2], b_reg[4];
+  auto fetch = [&](int k0) __attribute__((always_inline)) {
+    const bool inside = k0 + piece_k < k;
+    const int at = inside ? k0 + piece_k : 0;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      a_reg[i] = *reinterpret_cast<const ts_u32x4*>(a_src[i] + at);
+      if (!inside) a_reg[i] = ts_u32x4{0u, 0u, 0u, 0u};
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      b_reg[i] = load_once16(b_src[i] + at);
+      if (!inside) b_reg[i] = ts_u32x4{0u, 0u, 0u, 0u};
+    }
+  };
+  auto stage = [&]() __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+      *reinterpret_cast<ts_u32x4*>(a_tile + (piece_row + 32 * i) * MOE_LDS_ROW + piece_k) = a_reg[i];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      *reinterpret_cast<ts_u32x4*>(b_tile + (piece_row + 32 * i) * MOE_LDS_ROW + piece_k) = b_reg[i];
+  };
+
   moe_f32x4 acc[2][4];
 #pragma unroll
   for (int a = 0; a < 2; ++a)
 #pragma unroll
     for (int b = 0; b < 4; ++b) acc[a][b] = moe_f32x4{0.f, 0.f, 0.f, 0.f};
-  for (int k0 = 0; k0 < k; k0 += 32) {
-    ts_u32x4 af[2], bf[4];
+  fetch(0);
+  for (int k0 = 0; k0 < k; k0 += MOE_DEPTH) {
+    stage();
+    __syncthreads();
+    if (k0 + MOE_DEPTH < k) fetch(k0 + MOE_DEPTH);  // in flight while this iteration's products run
 #pragma unroll
-    for (int a = 0; a < 2; ++a) af[a] = *reinterpret_cast<const ts_u32x4*>(a_row[a] + k0);
+    for (int kk = 0; kk < MOE_DEPTH; kk += 32) {
+      ts_u32x4 af[2], bf[4];
 #pragma unroll
-    for (int b = 0; b < 4; ++b) bf[b] = *reinterpret_cast<const ts_u32x4*>(b_row[b] + k0);
-#pragma unroll
-    for (int a = 0; a < 2; ++a)
+      for (int a = 0; a < 2; ++a)
+        af[a] = *reinterpret_cast<const ts_u32x4*>(a_tile + (wm * 32 + 16 * a + r16) * MOE_LDS_ROW + kk + 8 * group);
 #pragma unroll
       for (int b = 0; b < 4; ++b)
-        acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(moe_bf16x8, af[a]),
-                                                            __builtin_bit_cast(moe_bf16x8, bf[b]), acc[a][b], 0, 0, 0);
+        bf[b] = *reinterpret_cast<const ts_u32x4*>(b_tile + (wn * 64 + 16 * b + r16) * MOE_LDS_ROW + kk + 8 * group);
+#pragma unroll
+      for (int a = 0; a < 2; ++a)
+#pragma unroll
+        for (int b = 0; b < 4; ++b)
+          acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(moe_bf16x8, af[a]),
+                                                              __builtin_bit_cast(moe_bf16x8, bf[b]), acc[a][b], 0, 0, 0);
+    }
+    __syncthreads();  // everyone has read this iteration's tiles before the next is staged
   }
-  // acc[a][b][i] is row 16 a + 4 group + i, column 16 b + r16 of the wavefront's tile.
+  // acc[a][b][i] is row 16 a + 4 group + i, column 16 b + r16 of the wavefront's 32 x 64.
 #pragma unroll
   for (int a = 0; a < 2; ++a) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const int r = row0 + 16 * a + 4 * group + i;
-      // The row's pair: held by the lane whose r16 is 4 group + i of the same a.
-      const int pair = __shfl(pair_of[a], 4 * group + i, 64);
+      const int r = rows_begin + wm * 32 + 16 * a + 4 * group + i;
+      const int pair = order[min(r, rows_end - 1)];
 #pragma unroll
       for (int b = 0; b < 4; ++b) {
-        const int col = col0 + 16 * b + r16;
+        const int col = col_begin + wn * 64 + 16 * b + r16;
         const float v = acc[a][b][i];
         if (GATED) {
           const float other = __shfl_xor(v, 1, 64);  // columns alternate gate, up
@@ -398,7 +422,7 @@ extern "C" int ts_moe_grouped_rows(void* out, const void* in, const void* weight
                                    hipStream_t stream) {
   if (pairs == 0) return TS_OK;
   if (!out || !in || !weight || !order || !tile_first || !row_first) return TS_ERR_ARG;
-  if (n < 1 || k < 32 || k % 32 != 0 || in_share < 1 || experts < 1 || experts > MOE_MAX_EXPERTS || (gated && (n & 1)))
+  if (n < 1 || k < 8 || k % 8 != 0 || in_share < 1 || experts < 1 || experts > MOE_MAX_EXPERTS || (gated && (n & 1)))
     return TS_ERR_SHAPE;
   if (((uintptr_t)in | (uintptr_t)weight) % 16 != 0) return TS_ERR_ARG;
   const GluRule rule = {steepness, limit, up_shift};

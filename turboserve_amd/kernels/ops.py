@@ -58,8 +58,8 @@ _SIGNATURES: dict[str, dict[str, list]] = {
         "ts_embed_positions": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
         "ts_copy_f32": [c_void_p, c_void_p, c_long, c_void_p],
         "ts_stream_offset": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
-        "ts_moe_route": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
-                         c_int, c_float, c_int, c_void_p],
+        "ts_moe_select": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float,
+                          c_void_p],
         "ts_moe_pair_rows": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float,
                              c_float, c_float, c_int, c_void_p],
         "ts_moe_group": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
@@ -609,29 +609,29 @@ class Ops:
     # -- routed feed-forward --------------------------------------------------------------------
 
     def moe_route(self, x: torch.Tensor, router: torch.Tensor, *, top: int, groups: int, keep: int, scale: float,
-                  extra: torch.Tensor | None = None) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor | None]:
-        """The router of a routed feed-forward, in 32-bit: ``s = sigmoid(router x)``; the experts
-        form ``groups`` equal groups of neighbours, a group's mark is the sum of its two largest
-        ``s``, only the ``keep`` best groups' experts can be taken, the ``top`` of them with the
-        largest ``s`` are.  Returns ``(taken [T, top] int32, weights [T, top] float32, gate)``:
-        weights are ``s / (sum of the taken s + 1e-20) * scale``; ``gate [T]`` is
-        ``sigmoid(extra . x)`` for a vector ``extra [H]`` (``None`` without one)."""
-        _gpu(x, router, extra)
+                  experts: int | None = None) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor | None]:
+        """The router of a routed feed-forward: ``z = x router^T`` by the engine's product with a
+        32-bit result, then in 32-bit ``s = sigmoid(z)``; the experts form ``groups`` equal groups
+        of neighbours, a group's mark is the sum of its two largest ``s``, only the ``keep`` best
+        groups' experts can be taken, the ``top`` of them with the largest ``s`` are.  Returns
+        ``(taken [T, top] int32, weights [T, top] float32, gate)``: weights are ``s / (sum of the
+        taken s + 1e-20) * scale``.  With ``experts`` one less than the rows of ``router``, the
+        last row is a gate's vector and ``gate [T]`` the sigmoid of its product (else ``None``)."""
+        _gpu(x, router)
         _need(x.dim() == 2 and x.is_contiguous() and router.dim() == 2 and router.is_contiguous()
               and router.shape[1] == x.shape[1] and router.dtype == x.dtype, "x [T, H] and router [E, H] of one dtype")
-        tokens, hidden = x.shape
-        experts = router.shape[0]
+        tokens = x.shape[0]
+        experts = router.shape[0] if experts is None else int(experts)
+        _need(router.shape[0] - experts in (0, 1), "the router holds the experts' rows and at most a gate's")
         _need(1 <= experts <= 1024 and 1 <= top <= 32 and groups >= 1 and experts % groups == 0 and 1 <= keep <= groups
               and top <= (experts // groups) * keep, "a routing rule the kernel does not take")
+        z = self.linear_float32_out(x, router)
+        _need(z.dtype == torch.float32 and z.stride(1) == 1, "the router's outputs must be 32-bit rows")
         taken = torch.empty((tokens, top), dtype=torch.int32, device=x.device)
         weights = torch.empty((tokens, top), dtype=torch.float32, device=x.device)
-        gate = None
-        if extra is not None:
-            _need(extra.numel() == hidden and extra.dtype == x.dtype and extra.is_contiguous(), "extra must be [H]")
-            gate = torch.empty((tokens,), dtype=torch.float32, device=x.device)
-        _check(self.core.ts_moe_route(_ptr(taken), _ptr(weights), _ptr(gate), _ptr(x), _ptr(router), _ptr(extra), tokens,
-                                      hidden, experts, top, groups, keep, float(scale), dtype_code(x.dtype), self.stream()),
-               "ts_moe_route")
+        gate = torch.empty((tokens,), dtype=torch.float32, device=x.device) if router.shape[0] > experts else None
+        _check(self.core.ts_moe_select(_ptr(taken), _ptr(weights), _ptr(gate), _ptr(z), tokens, z.stride(0), experts, top,
+                                       groups, keep, float(scale), self.stream()), "ts_moe_select")
         return taken, weights, gate
 
     def moe_pair_rows(self, rows: torch.Tensor, weight: torch.Tensor, taken: torch.Tensor, *, share: int,
@@ -664,12 +664,12 @@ class Ops:
 
     def moe_grouping(self, taken: torch.Tensor, experts: int, dtype: torch.dtype, *widths: int):
         """``(order, tile_first, row_first)`` for :meth:`moe_grouped_rows` where a step's pairs are
-        worth grouping by expert (bfloat16, many tokens, every inner width a multiple of 32), else
+        worth grouping by expert (bfloat16, many tokens, every inner width a multiple of 8), else
         ``None``.  All on the device: the host never sees who took which expert."""
         _gpu(taken)
         _i32(taken, "taken")
         if (dtype != torch.bfloat16 or taken.shape[0] < self.moe_grouped_min_tokens or experts > 1024
-                or any(w % 32 != 0 for w in widths)):
+                or any(w % 8 != 0 for w in widths)):
             return None
         pairs = taken.numel()
         order = torch.empty((pairs,), dtype=torch.int32, device=taken.device)
@@ -689,7 +689,7 @@ class Ops:
               and rows.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and rows.shape[1] == weight.shape[2],
               "rows [*, K] and weight [E, N, K] must be bfloat16")
         experts, n, k = weight.shape
-        _need(k % 32 == 0 and share >= 1 and rows.shape[0] * share >= pairs and order.numel() == pairs
+        _need(k % 8 == 0 and share >= 1 and rows.shape[0] * share >= pairs and order.numel() == pairs
               and tile_first.numel() == experts + 1, "grouping and sizes do not fit")
         if rule is not None:
             _need(n % 2 == 0, "a gated stack has an even number of rows")

@@ -72,7 +72,6 @@ class RoutedExperts(FeedForward):
         self.shared = None if shared is None else build_part("feed_forward", shared, self.name(shared_name), runtime)
         self.shared_gate_name = None if shared is None or not shared_gate_name else self.shared.name(shared_gate_name)
         self.router: torch.Tensor | None = None
-        self.shared_gate: torch.Tensor | None = None
         self.gate_up: torch.Tensor | None = None   # [E, 2 I, H], rows alternate gate, up
         self.down: torch.Tensor | None = None      # [E, H, I]
 
@@ -103,6 +102,9 @@ class RoutedExperts(FeedForward):
 
     def load(self, tensors: Mapping[str, torch.Tensor]) -> None:
         self.router = tensors[self.name(self.router_name)].contiguous()
+        if self.shared_gate_name:
+            # The shared expert's gate is one more row of the router's matrix: one product for both.
+            self.router = torch.cat([self.router, tensors[self.shared_gate_name].reshape(1, -1)], dim=0).contiguous()
         first = tensors[self._expert(0, 1)]
         self.gate_up = torch.empty((self.experts, 2 * self.expert_size, self.hidden_size), dtype=first.dtype, device=first.device)
         self.down = torch.empty((self.experts, self.hidden_size, self.expert_size), dtype=first.dtype, device=first.device)
@@ -113,13 +115,11 @@ class RoutedExperts(FeedForward):
         del first
         if self.shared is not None:
             self.shared.load(tensors)
-        if self.shared_gate_name:
-            self.shared_gate = tensors[self.shared_gate_name].reshape(-1).contiguous()
 
     def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
         ops = self.runtime.ops
         taken, weights, gate = ops.moe_route(x, self.router, top=self.top, groups=self.groups, keep=self.keep,
-                                             scale=self.route_scale, extra=self.shared_gate)
+                                             scale=self.route_scale, experts=self.experts)
         grouping = ops.moe_grouping(taken, self.experts, x.dtype, self.hidden_size, self.expert_size)
         units = ops.moe_expert_units(x, self.gate_up, taken, self.rule, grouping)
         outputs = ops.moe_expert_outputs(units, self.down, taken, grouping)
