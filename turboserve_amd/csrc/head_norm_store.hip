@@ -10,6 +10,8 @@
 // projection of type T this may be the projection itself), keys to key pages [NB, Hkv, BS, D] at
 // slot = page * BS + offset, values to the transposed value pages [NB, Hkv, Dv, BS].  A negative
 // slot or slots == nullptr: nothing is stored for that token.
+#include <type_traits>
+
 #include "common.hpp"
 
 #define HNS_MAX_DIM 512
@@ -104,6 +106,68 @@ head_norm_store_kernel(T* q_out, long q_stride, const P* proj, int splits, size_
   }
 }
 
+// The same for many tokens (prompt portions): bfloat16 in and out, no partial sums, no rotation,
+// head size a multiple of 8 and at most 128.  Sixteen lanes per (token, q or k head), eight
+// elements a lane with one 16-byte load and one 16-byte store; the sum of squares is formed over
+// the sixteen lanes of a row by data-parallel moves.  Per element the arithmetic of the kernel
+// above.
+__global__ void __launch_bounds__(256)
+head_norm_store_rows_kernel(bf16_t* q_out, long q_stride, const bf16_t* proj, bf16_t* __restrict__ k_pages,
+                            const bf16_t* __restrict__ q_gain, const bf16_t* __restrict__ k_gain, float eps,
+                            float gain_offset, const int* __restrict__ slots, int tokens, int heads, int kv_heads,
+                            int dim, int vdim, int block_size) {
+  const int qk_heads = heads + kv_heads;
+  const long items = (long)tokens * qk_heads;
+  const long asked = (long)blockIdx.x * 16 + threadIdx.x / 16;
+  const bool valid = asked < items;  // rows beyond the last item read the last item and store nothing
+  const long item = valid ? asked : items - 1;
+  const int piece = threadIdx.x % 16;
+  const int t = (int)(item / qk_heads), h = (int)(item % qk_heads);
+  const bool holds = piece * 8 < dim;
+  const size_t width = (size_t)qk_heads * dim + (size_t)kv_heads * vdim;
+  const bf16_t* row = proj + (size_t)t * width + (size_t)h * dim;
+  const bf16_t* gain = h < heads ? q_gain : k_gain;
+  ts_u32x4 raw = {0u, 0u, 0u, 0u}, graw = {0u, 0u, 0u, 0u};
+  if (holds) {
+    raw = *reinterpret_cast<const ts_u32x4*>(row + piece * 8);
+    if (gain) graw = *reinterpret_cast<const ts_u32x4*>(gain + piece * 8);
+  }
+  float x[8], g[8];
+  float ss = 0.f;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    x[2 * e] = __uint_as_float(raw[e] << 16);
+    x[2 * e + 1] = __uint_as_float(raw[e] & 0xffff0000u);
+    g[2 * e] = __uint_as_float(graw[e] << 16);
+    g[2 * e + 1] = __uint_as_float(graw[e] & 0xffff0000u);
+    ss += x[2 * e] * x[2 * e] + x[2 * e + 1] * x[2 * e + 1];
+  }
+  if (gain) {
+    // Over the row of sixteen lanes (the first four steps of wave_sum).
+    ss += lanes_moved<0xB1, 0xF>(0.f, ss);
+    ss += lanes_moved<0x4E, 0xF>(0.f, ss);
+    ss += lanes_moved<0x141, 0xF>(0.f, ss);
+    ss += lanes_moved<0x140, 0xF>(0.f, ss);
+    const float r = rsqrtf(ss / (float)dim + eps);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x[e] = x[e] * r * (gain_offset + g[e]);
+  }
+  bf16_t* dst = nullptr;
+  if (h < heads) {
+    dst = q_out + (size_t)t * q_stride + (size_t)h * dim;
+  } else {
+    const int slot = slots ? slots[t] : -1;
+    if (slot >= 0)
+      dst = k_pages + (((size_t)(slot / block_size) * kv_heads + (h - heads)) * block_size + slot % block_size) * dim;
+  }
+  if (!dst || !holds || !valid) return;
+  ts_u32x4 packed;
+#pragma unroll
+  for (int e = 0; e < 4; ++e)
+    packed[e] = (uint32_t)from_float<bf16_t>(x[2 * e]).bits | ((uint32_t)from_float<bf16_t>(x[2 * e + 1]).bits << 16);
+  *reinterpret_cast<ts_u32x4*>(dst + piece * 8) = packed;
+}
+
 // Values: one block per (group of 8 consecutive tokens, KV head); a thread collects one value
 // dimension of the 8 tokens.  Where the group's slots are 8 consecutive ones that start at a
 // multiple of 8 inside one page, a bfloat16 group leaves as one 16-byte store.
@@ -170,6 +234,14 @@ static void launch_head_norm_store(void* q_out, long q_stride, const void* proj,
                                    const int* positions, const int* slots, int tokens, int heads, int kv_heads,
                                    int dim, int vdim, int block_size, hipStream_t stream) {
   const long items = (long)tokens * (heads + kv_heads);
+  const bool aligned = ((uintptr_t)q_out | (uintptr_t)proj | (uintptr_t)k_pages | (uintptr_t)q_gain | (uintptr_t)k_gain) % 16 == 0 &&
+                       q_stride % 8 == 0 && vdim % 8 == 0;
+  if (std::is_same<T, bf16_t>::value && std::is_same<P, bf16_t>::value && splits == 1 && !cos_table && dim % 8 == 0 &&
+      dim <= 128 && tokens >= 4 * HNS_GROUP && aligned)
+    hipLaunchKernelGGL(head_norm_store_rows_kernel, dim3((unsigned)((items + 15) / 16)), dim3(256), 0, stream, (bf16_t*)q_out,
+                       q_stride, (const bf16_t*)proj, (bf16_t*)k_pages, (const bf16_t*)q_gain, (const bf16_t*)k_gain, eps,
+                       gain_offset, slots, tokens, heads, kv_heads, dim, vdim, block_size);
+  else
   hipLaunchKernelGGL((head_norm_store_kernel<T, P>), dim3((unsigned)((items + HNS_WAVES - 1) / HNS_WAVES)),
                      dim3(64 * HNS_WAVES), 0, stream, (T*)q_out, q_stride, (const P*)proj, splits, (size_t)split_stride,
                      (T*)k_pages, (const T*)q_gain, (const T*)k_gain, eps, gain_offset, cos_table, sin_table, positions,

@@ -248,7 +248,7 @@ extern "C" int ts_moe_combine(float* out, const float* pair_out, const float* we
 // columns), found from tile_first; blocks beyond the last tile leave at once, so the grid is the
 // upper bound P / MOE_TILE_ROWS + E.  K must be a multiple of 8.
 // ---------------------------------------------------------------------------------------------
-#define MOE_TILE_ROWS 64
+#define MOE_TILE_ROWS 128
 #define MOE_TILE_COLS 128
 
 __global__ void __launch_bounds__(1024)
@@ -296,10 +296,11 @@ typedef float moe_f32x4 __attribute__((ext_vector_type(4)));
 #define MOE_DEPTH 64                   // k per iteration
 #define MOE_LDS_ROW (MOE_DEPTH + 8)    // elements; 144 bytes: sixteen rows' same piece lies in sixteen different banks' quads
 
-// A block of four wavefronts owns 64 sorted rows x 128 columns; per iteration both operands go
+// A block of four wavefronts owns 128 sorted rows x 128 columns; per iteration both operands go
 // global memory -> registers (16-byte pieces, eight consecutive threads a row's 128 bytes) -> LDS ->
 // matrix cores, and the loads of the next iteration are in flight while this one's products run.
-// A wavefront computes 32 rows x 64 columns (2 x 4 tiles of 16 x 16).
+// A wavefront computes 64 rows x 64 columns (4 x 4 tiles of 16 x 16: a fragment read from LDS
+// serves four matrix instructions).
 template <bool GATED>
 __global__ void __launch_bounds__(256)
 moe_grouped_rows_kernel(void* __restrict__ out_any, const bf16_t* __restrict__ in, const bf16_t* __restrict__ weight,
@@ -332,21 +333,21 @@ moe_grouped_rows_kernel(void* __restrict__ out_any, const bf16_t* __restrict__ i
   // What this thread fetches per iteration: pieces tid + 256 i of the tiles, piece = (row, 8 k).
   const int piece_k = 8 * (tid % 8);
   const int piece_row = tid / 8;  // + 32 i
-  const bf16_t* a_src[2];
+  const bf16_t* a_src[4];
   const bf16_t* b_src[4];
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
+  for (int i = 0; i < 4; ++i) {
     const int r = min(rows_begin + piece_row + 32 * i, rows_end - 1);
     a_src[i] = in + (size_t)(order[r] / in_share) * k;
   }
 #pragma unroll
   for (int i = 0; i < 4; ++i) b_src[i] = w + (size_t)min(col_begin + piece_row + 32 * i, n - 1) * k;
-  ts_u32x4 a_reg[2], b_reg[4];
+  ts_u32x4 a_reg[4], b_reg[4];
   auto fetch = [&](int k0) __attribute__((always_inline)) {
     const bool inside = k0 + piece_k < k;
     const int at = inside ? k0 + piece_k : 0;
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < 4; ++i) {
       a_reg[i] = *reinterpret_cast<const ts_u32x4*>(a_src[i] + at);
       if (!inside) a_reg[i] = ts_u32x4{0u, 0u, 0u, 0u};
     }
@@ -358,16 +359,16 @@ moe_grouped_rows_kernel(void* __restrict__ out_any, const bf16_t* __restrict__ i
   };
   auto stage = [&]() __attribute__((always_inline)) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < 4; ++i)
       *reinterpret_cast<ts_u32x4*>(a_tile + (piece_row + 32 * i) * MOE_LDS_ROW + piece_k) = a_reg[i];
 #pragma unroll
     for (int i = 0; i < 4; ++i)
       *reinterpret_cast<ts_u32x4*>(b_tile + (piece_row + 32 * i) * MOE_LDS_ROW + piece_k) = b_reg[i];
   };
 
-  moe_f32x4 acc[2][4];
+  moe_f32x4 acc[4][4];
 #pragma unroll
-  for (int a = 0; a < 2; ++a)
+  for (int a = 0; a < 4; ++a)
 #pragma unroll
     for (int b = 0; b < 4; ++b) acc[a][b] = moe_f32x4{0.f, 0.f, 0.f, 0.f};
   fetch(0);
@@ -377,15 +378,15 @@ moe_grouped_rows_kernel(void* __restrict__ out_any, const bf16_t* __restrict__ i
     if (k0 + MOE_DEPTH < k) fetch(k0 + MOE_DEPTH);  // in flight while this iteration's products run
 #pragma unroll
     for (int kk = 0; kk < MOE_DEPTH; kk += 32) {
-      ts_u32x4 af[2], bf[4];
+      ts_u32x4 af[4], bf[4];
 #pragma unroll
-      for (int a = 0; a < 2; ++a)
-        af[a] = *reinterpret_cast<const ts_u32x4*>(a_tile + (wm * 32 + 16 * a + r16) * MOE_LDS_ROW + kk + 8 * group);
+      for (int a = 0; a < 4; ++a)
+        af[a] = *reinterpret_cast<const ts_u32x4*>(a_tile + (wm * 64 + 16 * a + r16) * MOE_LDS_ROW + kk + 8 * group);
 #pragma unroll
       for (int b = 0; b < 4; ++b)
         bf[b] = *reinterpret_cast<const ts_u32x4*>(b_tile + (wn * 64 + 16 * b + r16) * MOE_LDS_ROW + kk + 8 * group);
 #pragma unroll
-      for (int a = 0; a < 2; ++a)
+      for (int a = 0; a < 4; ++a)
 #pragma unroll
         for (int b = 0; b < 4; ++b)
           acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(moe_bf16x8, af[a]),
@@ -393,12 +394,12 @@ moe_grouped_rows_kernel(void* __restrict__ out_any, const bf16_t* __restrict__ i
     }
     __syncthreads();  // everyone has read this iteration's tiles before the next is staged
   }
-  // acc[a][b][i] is row 16 a + 4 group + i, column 16 b + r16 of the wavefront's 32 x 64.
+  // acc[a][b][i] is row 16 a + 4 group + i, column 16 b + r16 of the wavefront's 64 x 64.
 #pragma unroll
-  for (int a = 0; a < 2; ++a) {
+  for (int a = 0; a < 4; ++a) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const int r = rows_begin + wm * 32 + 16 * a + 4 * group + i;
+      const int r = rows_begin + wm * 64 + 16 * a + 4 * group + i;
       const int pair = order[min(r, rows_end - 1)];
 #pragma unroll
       for (int b = 0; b < 4; ++b) {
