@@ -262,6 +262,17 @@ def test_mixed_batches_on_pages_that_are_used_again(case, dtype):
     check_against_plain(case, dtype, steps)
 
 
+def test_long_decoding(case):
+    """One short prompt, then 150 tokens one by one (recorded steps whose tables grow past
+    several widths), in 32-bit."""
+    name, config = case["name"], st.TINY[case["name"]][0]
+    tokens = st_tokens(config["vocab"], 156, 4242)
+    requests = {"long": tokens}
+    steps = th.prefix_then_single(requests, tail=150)
+    got = th.collect(steps, run_trace(case["folders"]["float32"], "float32", case["page"], steps), requests)["long"]
+    assert excess(got, st.plain_logits(case["folders"]["float32"], tokens), "float32") <= 1.0, name
+
+
 def test_cuttings_agree_in_32_bit(case):
     """The logits of a position do not depend on how its request was cut or batched."""
     folder, page = case["folders"]["float32"], case["page"]

@@ -102,3 +102,17 @@ def test_the_position_vectors():
     assert torch.allclose(rows[1, 2:4], torch.tensor([torch.sin(torch.tensor(3 * rate)), torch.cos(torch.tensor(3 * rate))]))
     from turboserve_amd.parts.ends import sinusoid_table
     assert torch.allclose(sinusoid_table(40, 7, 10000.0), plain.sinusoid_rows(range(40), 7), atol=1e-6)
+
+
+def test_a_random_model_folder_is_written_and_read_back(tmp_path):
+    from turboserve_amd.config.model_config import read_config_json
+    from turboserve_amd.weights.random_init import write_random_model
+
+    folder = write_random_model(st.CONFIG_Q, tmp_path / "model", seed=3, dtype=torch.bfloat16, std=0.05)
+    assert parse_model_config(read_config_json(folder)) == parse_model_config(st.CONFIG_Q)
+    config, tensors = st.read_model_dir(folder)
+    _, model = describe_model(config)
+    assert set(tensors) == set(model.tensor_specs())
+    assert float(tensors["l0.norm1"].abs().max()) == 0.0 and float(tensors["l0.mix.q.norm"].min()) == 1.0
+    logits = plain.forward(config, tensors, [5, 1, 96, 40])
+    assert logits.shape == (4, 97) and bool(torch.isfinite(logits).all())

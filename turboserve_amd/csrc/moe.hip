@@ -298,7 +298,8 @@ typedef float moe_f32x4 __attribute__((ext_vector_type(4)));
 
 // A block of four wavefronts owns 128 sorted rows x 128 columns; per iteration both operands go
 // global memory -> registers (16-byte pieces, eight consecutive threads a row's 128 bytes) -> LDS ->
-// matrix cores, and the loads of the next iteration are in flight while this one's products run.
+// matrix cores.  Two LDS buffers: the loads of the next iteration are in flight while this one's
+// products run and go into the other buffer right behind them, so an iteration has one barrier.
 // A wavefront computes 64 rows x 64 columns (4 x 4 tiles of 16 x 16: a fragment read from LDS
 // serves four matrix instructions).
 template <bool GATED>
@@ -306,8 +307,8 @@ __global__ void __launch_bounds__(256)
 moe_grouped_rows_kernel(void* __restrict__ out_any, const bf16_t* __restrict__ in, const bf16_t* __restrict__ weight,
                         const int* __restrict__ order, const int* __restrict__ tile_first,
                         const int* __restrict__ row_first, int in_share, int n, int k, int experts, GluRule rule) {
-  __shared__ __attribute__((aligned(16))) uint16_t a_tile[MOE_TILE_ROWS * MOE_LDS_ROW];
-  __shared__ __attribute__((aligned(16))) uint16_t b_tile[MOE_TILE_COLS * MOE_LDS_ROW];
+  extern __shared__ __attribute__((aligned(16))) uint16_t moe_tiles[];  // [2][rows of A, then rows of B][MOE_LDS_ROW]
+  constexpr int BUFFER = (MOE_TILE_ROWS + MOE_TILE_COLS) * MOE_LDS_ROW;
   __shared__ int found;
   const int tile = blockIdx.x;
   if (tile >= tile_first[experts]) return;  // the whole block leaves together
@@ -357,7 +358,9 @@ moe_grouped_rows_kernel(void* __restrict__ out_any, const bf16_t* __restrict__ i
       if (!inside) b_reg[i] = ts_u32x4{0u, 0u, 0u, 0u};
     }
   };
-  auto stage = [&]() __attribute__((always_inline)) {
+  auto stage = [&](int buffer) __attribute__((always_inline)) {
+    uint16_t* a_tile = moe_tiles + buffer * BUFFER;
+    uint16_t* b_tile = a_tile + MOE_TILE_ROWS * MOE_LDS_ROW;
 #pragma unroll
     for (int i = 0; i < 4; ++i)
       *reinterpret_cast<ts_u32x4*>(a_tile + (piece_row + 32 * i) * MOE_LDS_ROW + piece_k) = a_reg[i];
@@ -372,10 +375,13 @@ moe_grouped_rows_kernel(void* __restrict__ out_any, const bf16_t* __restrict__ i
 #pragma unroll
     for (int b = 0; b < 4; ++b) acc[a][b] = moe_f32x4{0.f, 0.f, 0.f, 0.f};
   fetch(0);
-  for (int k0 = 0; k0 < k; k0 += MOE_DEPTH) {
-    stage();
-    __syncthreads();
-    if (k0 + MOE_DEPTH < k) fetch(k0 + MOE_DEPTH);  // in flight while this iteration's products run
+  stage(0);
+  __syncthreads();
+  for (int k0 = 0, it = 0; k0 < k; k0 += MOE_DEPTH, ++it) {
+    const bool more = k0 + MOE_DEPTH < k;
+    if (more) fetch(k0 + MOE_DEPTH);  // in flight while this iteration's products run
+    const uint16_t* a_tile = moe_tiles + (it & 1) * BUFFER;
+    const uint16_t* b_tile = a_tile + MOE_TILE_ROWS * MOE_LDS_ROW;
 #pragma unroll
     for (int kk = 0; kk < MOE_DEPTH; kk += 32) {
       ts_u32x4 af[4], bf[4];
@@ -392,7 +398,10 @@ moe_grouped_rows_kernel(void* __restrict__ out_any, const bf16_t* __restrict__ i
           acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(moe_bf16x8, af[a]),
                                                               __builtin_bit_cast(moe_bf16x8, bf[b]), acc[a][b], 0, 0, 0);
     }
-    __syncthreads();  // everyone has read this iteration's tiles before the next is staged
+    // The other buffer was last read in the iteration before this one, which every wavefront
+    // left through the barrier below.
+    if (more) stage((it + 1) & 1);
+    __syncthreads();
   }
   // acc[a][b][i] is row 16 a + 4 group + i, column 16 b + r16 of the wavefront's 64 x 64.
 #pragma unroll
@@ -429,9 +438,18 @@ extern "C" int ts_moe_grouped_rows(void* out, const void* in, const void* weight
   const GluRule rule = {steepness, limit, up_shift};
   const dim3 grid(pairs / MOE_TILE_ROWS + experts + 1, (n + MOE_TILE_COLS - 1) / MOE_TILE_COLS), block(256);
   if (grid.y > 65535) return TS_ERR_SHAPE;
+  constexpr size_t lds = (size_t)2 * (MOE_TILE_ROWS + MOE_TILE_COLS) * MOE_LDS_ROW * sizeof(uint16_t);
+  static_assert(lds <= 80 * 1024, "two workgroups' buffers fit a compute unit's LDS");
+  static bool raised = false;  // per process; the attribute belongs to the kernels
+  if (!raised) {
+    if (hipFuncSetAttribute((const void*)moe_grouped_rows_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess ||
+        hipFuncSetAttribute((const void*)moe_grouped_rows_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+      return TS_ERR_LAUNCH;
+    raised = true;
+  }
   if (gated)
-    hipLaunchKernelGGL(moe_grouped_rows_kernel<true>, grid, block, 0, stream, out, (const bf16_t*)in, (const bf16_t*)weight, order, tile_first, row_first, in_share, n, k, experts, rule);
+    hipLaunchKernelGGL(moe_grouped_rows_kernel<true>, grid, block, lds, stream, out, (const bf16_t*)in, (const bf16_t*)weight, order, tile_first, row_first, in_share, n, k, experts, rule);
   else
-    hipLaunchKernelGGL(moe_grouped_rows_kernel<false>, grid, block, 0, stream, out, (const bf16_t*)in, (const bf16_t*)weight, order, tile_first, row_first, in_share, n, k, experts, rule);
+    hipLaunchKernelGGL(moe_grouped_rows_kernel<false>, grid, block, lds, stream, out, (const bf16_t*)in, (const bf16_t*)weight, order, tile_first, row_first, in_share, n, k, experts, rule);
   return ts_launch_status();
 }
