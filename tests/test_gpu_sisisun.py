@@ -5,7 +5,11 @@ through the engine's own entry point."""
 
 from __future__ import annotations
 
-import copy
+import json
+import random
+import subprocess
+import sys
+from pathlib import Path
 
 import pytest
 import torch
@@ -17,6 +21,7 @@ from plain import sisisun_plain as plain
 pytestmark = pytest.mark.gpu
 
 DEV = "cuda:0"
+ROOT = Path(__file__).resolve().parent.parent
 #: 32-bit engine against the 32-bit plain implementation, relative to a position's largest logit.
 RTOL_F32 = 2e-4
 #: bfloat16 engine (weights stored in bfloat16) against the plain implementation in 32-bit on the
@@ -283,6 +288,96 @@ def test_cuttings_agree_in_32_bit(case):
         for rid, base in results["whole"].items():
             scale = base.abs().amax(dim=-1, keepdim=True).clamp_min(1.0)
             assert float(((got[rid] - base).abs() / scale).max()) <= 2e-5, (name, rid)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_the_replay_program(case, dtype, tmp_path):
+    """``bin/trace_run`` itself on a model folder of this design: JSON lines in, ``done`` lines and
+    .f32 files out, steps that want nothing included."""
+    if case["name"] != "P":
+        pytest.skip("one configuration is enough for the subprocess test")
+    steps = th.mixed(case["requests"], (7, 2, 19, 32, 3), max_live=3, decode_tail=9)
+    for record in steps[1::3]:  # every third step wants nothing: the program waits for none of its results
+        for entry in record["entries"]:
+            entry["want"] = []
+    out = tmp_path / "out"
+    proc = subprocess.run(
+        [sys.executable, str(ROOT / "bin" / "trace_run"), "--model", str(case["folders"][dtype]), "--dtype", dtype,
+         "--out", str(out), "--max-tokens", str(th.peak_tokens(steps)), "--page-size", str(case["page"])],
+        input="".join(json.dumps(s) + "\n" for s in steps), capture_output=True, text=True, timeout=600,
+    )
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert [line for line in proc.stdout.splitlines() if line.startswith("done ")] == [f"done {s['step']}" for s in steps]
+    import numpy as np
+
+    vocab = st.TINY["P"][0]["vocab"]
+    position = {rid: 0 for rid in case["requests"]}
+    for record in steps:
+        wanted = sum(len(e["want"]) for e in record["entries"])
+        path = out / f"{record['step']}.f32"
+        assert path.exists() == bool(wanted)
+        got = torch.from_numpy(np.fromfile(path, dtype="<f4").reshape(wanted, vocab).copy()) if wanted else None
+        row = 0
+        for entry in record["entries"]:
+            for place in entry["want"]:
+                want = case["expected"][dtype][entry["id"]][position[entry["id"]] + place]
+                assert excess(got[row:row + 1], want[None], dtype) <= (1.0 if dtype == "float32" else BF16_OUTLIERS)
+                row += 1
+            position[entry["id"]] += len(entry["tokens"])
+
+
+def random_config(rng: random.Random) -> dict:
+    width = rng.choice([40, 52, 64, 72, 96, 100, 128, 160, 192])
+    layers = []
+    for _ in range(rng.randint(1, 4)):
+        kv = rng.choice([1, 1, 2, 3, 4])
+        heads = kv * rng.choice([1, 1, 2, 3, 4, 8])
+        dim = rng.choice([8, 12, 16, 20, 24, 32, 40, 48, 64, 80, 96, 128])
+        vdim = dim if rng.random() < 0.6 else rng.choice([8, 12, 16, 24, 32, 48, 64, 72])
+        mixer = st.attention(heads, kv, dim, vdim, rng.choice([3.0, 10.0, 20.0, 50.0]), scale=rng.choice([dim ** -0.5, 0.2, 0.5]))
+        kind = rng.choice(["dense", "moe", "moe", "none"])
+        mlp = None
+        if kind == "dense":
+            mlp = st.dense(rng.choice([24, 44, 64, 100, 256]), rng.choice([0.5, 2.0, 7.0]))
+        elif kind == "moe":
+            count, size = rng.choice([1, 2, 3, 4]), rng.choice([1, 2, 3, 4, 8])
+            keep = rng.randint(1, count)
+            mlp = st.moe(count * size, rng.randint(1, min(size * keep, 6)), count, keep, rng.choice([1.0, 2.5]),
+                         rng.choice([16, 28, 32, 40, 96]), rng.choice([0, 0, 24, 64]))
+        layers.append(st.layer(mixer, mlp))
+    start = rng.randint(0, len(layers))
+    return {"architecture": "Sisisun", "vocab": rng.choice([50, 97, 256, 333]), "width": width,
+            "norm": {"eps": rng.choice([1e-6, 1e-5])}, "layers": layers,
+            "loop": {"start": start, "stop": rng.randint(start, len(layers)), "times": rng.randint(1, 3)}}
+
+
+@pytest.mark.parametrize("trial", range(12))
+def test_random_configurations_replay_like_plain(trial, tmp_path):
+    """Seeded random configurations: one to five layers in any order, loops that are empty, whole
+    or partial, head sizes that the matrix-core kernels take and ones they do not, values
+    narrower and wider than keys, experts in one group or many, widths and feed-forwards that
+    16-byte accesses do not divide; whole, token by token and mixed, in 32-bit (every position
+    inside the bound) and in bfloat16 (nine positions in ten inside it: a token that two experts
+    score alike may go either way there)."""
+    rng = random.Random(7000 + trial)
+    config = random_config(rng)
+    lengths = [rng.randint(1, 6), rng.randint(10, 60), rng.randint(100, 260), rng.randint(20, 90)]
+    requests = {f"r{i}": [rng.randrange(config["vocab"]) for _ in range(n)] for i, n in enumerate(lengths)}
+    for dtype, stored, std in (("float32", torch.float32, 0.15), ("bfloat16", torch.bfloat16, 0.06)):
+        folder = st.make_model_dir(tmp_path / dtype, config, trial, stored, std=std)
+        want = {rid: st.plain_logits(folder, tokens) for rid, tokens in requests.items()}
+        ways = (th.whole(requests), th.prefix_then_single(requests, tail=20),
+                th.mixed(requests, (7, 2, 40, 150, 3), max_live=4, decode_tail=5))
+        for steps in ways:
+            outputs = run_trace(folder, dtype, 16, steps, max_tokens=th.peak_tokens(steps))
+            got = th.collect(steps, outputs, requests)
+            for rid in requests:
+                if dtype == "float32":
+                    assert excess(got[rid], want[rid], dtype) <= 1.0, (trial, rid, config)
+                else:
+                    bound = RTOL_BF16 * want[rid].abs().amax(dim=-1).clamp_min(1.0)
+                    rows = (got[rid] - want[rid]).abs().amax(dim=-1) / bound
+                    assert float(rows.sort().values[int(0.9 * (len(rows) - 1))]) <= 1.0, (trial, rid, config)
 
 
 # ---------------------------------------------------------------------------------------------
