@@ -293,24 +293,33 @@ extern "C" int ts_moe_group(int* order, int* tile_first, int* row_first, const i
 typedef __bf16 moe_bf16x8 __attribute__((ext_vector_type(8)));
 typedef float moe_f32x4 __attribute__((ext_vector_type(4)));
 
-#define MOE_DEPTH 64                   // k per iteration
-#define MOE_LDS_ROW (MOE_DEPTH + 8)    // elements; 144 bytes: sixteen rows' same piece lies in sixteen different banks' quads
+#define MOE_DEPTH 128                  // k per iteration
+#define MOE_LDS_ROW (MOE_DEPTH + 8)    // elements; 272 bytes: sixteen rows' same piece lies in sixteen different banks' quads
 
 // A block of four wavefronts owns 128 sorted rows x 128 columns; per iteration both operands go
 // global memory -> registers (16-byte pieces, eight consecutive threads a row's 128 bytes) -> LDS ->
-// matrix cores.  Two LDS buffers: the loads of the next iteration are in flight while this one's
-// products run and go into the other buffer right behind them, so an iteration has one barrier.
+// matrix cores, 128 of K per iteration; the loads of the next iteration (sixteen 16-byte pieces a
+// thread) are in flight while this one's products run: what an iteration waits for is a trip
+// to memory, so it carries as many bytes as the registers hold.
 // A wavefront computes 64 rows x 64 columns (4 x 4 tiles of 16 x 16: a fragment read from LDS
 // serves four matrix instructions).
 template <bool GATED>
 __global__ void __launch_bounds__(256)
 moe_grouped_rows_kernel(void* __restrict__ out_any, const bf16_t* __restrict__ in, const bf16_t* __restrict__ weight,
                         const int* __restrict__ order, const int* __restrict__ tile_first,
-                        const int* __restrict__ row_first, int in_share, int n, int k, int experts, GluRule rule) {
-  extern __shared__ __attribute__((aligned(16))) uint16_t moe_tiles[];  // [2][rows of A, then rows of B][MOE_LDS_ROW]
-  constexpr int BUFFER = (MOE_TILE_ROWS + MOE_TILE_COLS) * MOE_LDS_ROW;
+                        const int* __restrict__ row_first, int in_share, int n, int k, int experts, GluRule rule,
+                        int tile_slots, int col_tiles) {
+  extern __shared__ __attribute__((aligned(16))) uint16_t moe_tiles[];  // [rows of A, then rows of B][MOE_LDS_ROW]
   __shared__ int found;
-  const int tile = blockIdx.x;
+  // Workgroup id -> (row tile, column tile): consecutive ids go to the eight dies in turn, so a
+  // die's ids are id % 8 == die; of those, consecutive ones take consecutive row tiles under one
+  // column tile, so the row tiles of an expert, which share their weights, meet in one die's L2.
+  const int total = tile_slots * col_tiles;
+  const int per_die = (total + 7) / 8;
+  const int logical = (int)(blockIdx.x % 8) * per_die + (int)(blockIdx.x / 8);
+  if (logical >= total) return;
+  const int tile = logical % tile_slots;
+  const int col_tile = logical / tile_slots;
   if (tile >= tile_first[experts]) return;  // the whole block leaves together
   if (threadIdx.x < TS_WAVE) {
     // The expert whose tiles hold this one.
@@ -328,45 +337,49 @@ moe_grouped_rows_kernel(void* __restrict__ out_any, const bf16_t* __restrict__ i
   const int wm = wave / 2, wn = wave % 2;
   const int rows_begin = row_first[e] + (tile - tile_first[e]) * MOE_TILE_ROWS;
   const int rows_end = row_first[e + 1];
-  const int col_begin = blockIdx.y * MOE_TILE_COLS;
+  const int col_begin = col_tile * MOE_TILE_COLS;
   const bf16_t* w = weight + (size_t)e * n * k;
 
   // What this thread fetches per iteration: pieces tid + 256 i of the tiles, piece = (row, 8 k).
-  const int piece_k = 8 * (tid % 8);
-  const int piece_row = tid / 8;  // + 32 i
-  const bf16_t* a_src[4];
-  const bf16_t* b_src[4];
+  constexpr int ROW_PIECES = MOE_DEPTH / 8;     // 16-byte pieces of a row of an iteration
+  constexpr int PASS_ROWS = 256 / ROW_PIECES;   // rows one pass of the threads covers
+  constexpr int PASSES = MOE_TILE_ROWS / PASS_ROWS;
+  static_assert(MOE_TILE_ROWS == MOE_TILE_COLS, "both tiles take the same passes");
+  const int piece_k = 8 * (tid % ROW_PIECES);
+  const int piece_row = tid / ROW_PIECES;  // + PASS_ROWS i
+  const bf16_t* a_src[PASSES];
+  const bf16_t* b_src[PASSES];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int r = min(rows_begin + piece_row + 32 * i, rows_end - 1);
+  for (int i = 0; i < PASSES; ++i) {
+    const int r = min(rows_begin + piece_row + PASS_ROWS * i, rows_end - 1);
     a_src[i] = in + (size_t)(order[r] / in_share) * k;
   }
 #pragma unroll
-  for (int i = 0; i < 4; ++i) b_src[i] = w + (size_t)min(col_begin + piece_row + 32 * i, n - 1) * k;
-  ts_u32x4 a_reg[4], b_reg[4];
+  for (int i = 0; i < PASSES; ++i) b_src[i] = w + (size_t)min(col_begin + piece_row + PASS_ROWS * i, n - 1) * k;
+  ts_u32x4 a_reg[PASSES], b_reg[PASSES];
   auto fetch = [&](int k0) __attribute__((always_inline)) {
     const bool inside = k0 + piece_k < k;
     const int at = inside ? k0 + piece_k : 0;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < PASSES; ++i) {
       a_reg[i] = *reinterpret_cast<const ts_u32x4*>(a_src[i] + at);
       if (!inside) a_reg[i] = ts_u32x4{0u, 0u, 0u, 0u};
     }
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      b_reg[i] = load_once16(b_src[i] + at);
+    for (int i = 0; i < PASSES; ++i) {
+      b_reg[i] = *reinterpret_cast<const ts_u32x4*>(b_src[i] + at);  // plain: other row tiles read it again
       if (!inside) b_reg[i] = ts_u32x4{0u, 0u, 0u, 0u};
     }
   };
-  auto stage = [&](int buffer) __attribute__((always_inline)) {
-    uint16_t* a_tile = moe_tiles + buffer * BUFFER;
-    uint16_t* b_tile = a_tile + MOE_TILE_ROWS * MOE_LDS_ROW;
+  uint16_t* a_tile = moe_tiles;
+  uint16_t* b_tile = a_tile + MOE_TILE_ROWS * MOE_LDS_ROW;
+  auto stage = [&]() __attribute__((always_inline)) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-      *reinterpret_cast<ts_u32x4*>(a_tile + (piece_row + 32 * i) * MOE_LDS_ROW + piece_k) = a_reg[i];
+    for (int i = 0; i < PASSES; ++i)
+      *reinterpret_cast<ts_u32x4*>(a_tile + (piece_row + PASS_ROWS * i) * MOE_LDS_ROW + piece_k) = a_reg[i];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-      *reinterpret_cast<ts_u32x4*>(b_tile + (piece_row + 32 * i) * MOE_LDS_ROW + piece_k) = b_reg[i];
+    for (int i = 0; i < PASSES; ++i)
+      *reinterpret_cast<ts_u32x4*>(b_tile + (piece_row + PASS_ROWS * i) * MOE_LDS_ROW + piece_k) = b_reg[i];
   };
 
   moe_f32x4 acc[4][4];
@@ -375,13 +388,10 @@ moe_grouped_rows_kernel(void* __restrict__ out_any, const bf16_t* __restrict__ i
 #pragma unroll
     for (int b = 0; b < 4; ++b) acc[a][b] = moe_f32x4{0.f, 0.f, 0.f, 0.f};
   fetch(0);
-  stage(0);
-  __syncthreads();
-  for (int k0 = 0, it = 0; k0 < k; k0 += MOE_DEPTH, ++it) {
-    const bool more = k0 + MOE_DEPTH < k;
-    if (more) fetch(k0 + MOE_DEPTH);  // in flight while this iteration's products run
-    const uint16_t* a_tile = moe_tiles + (it & 1) * BUFFER;
-    const uint16_t* b_tile = a_tile + MOE_TILE_ROWS * MOE_LDS_ROW;
+  for (int k0 = 0; k0 < k; k0 += MOE_DEPTH) {
+    stage();
+    __syncthreads();
+    if (k0 + MOE_DEPTH < k) fetch(k0 + MOE_DEPTH);  // in flight while this iteration's products run
 #pragma unroll
     for (int kk = 0; kk < MOE_DEPTH; kk += 32) {
       ts_u32x4 af[4], bf[4];
@@ -398,10 +408,7 @@ moe_grouped_rows_kernel(void* __restrict__ out_any, const bf16_t* __restrict__ i
           acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(moe_bf16x8, af[a]),
                                                               __builtin_bit_cast(moe_bf16x8, bf[b]), acc[a][b], 0, 0, 0);
     }
-    // The other buffer was last read in the iteration before this one, which every wavefront
-    // left through the barrier below.
-    if (more) stage((it + 1) & 1);
-    __syncthreads();
+    __syncthreads();  // everyone has read this iteration's tiles before the next is staged
   }
   // acc[a][b][i] is row 16 a + 4 group + i, column 16 b + r16 of the wavefront's 64 x 64.
 #pragma unroll
@@ -436,9 +443,10 @@ extern "C" int ts_moe_grouped_rows(void* out, const void* in, const void* weight
     return TS_ERR_SHAPE;
   if (((uintptr_t)in | (uintptr_t)weight) % 16 != 0) return TS_ERR_ARG;
   const GluRule rule = {steepness, limit, up_shift};
-  const dim3 grid(pairs / MOE_TILE_ROWS + experts + 1, (n + MOE_TILE_COLS - 1) / MOE_TILE_COLS), block(256);
-  if (grid.y > 65535) return TS_ERR_SHAPE;
-  constexpr size_t lds = (size_t)2 * (MOE_TILE_ROWS + MOE_TILE_COLS) * MOE_LDS_ROW * sizeof(uint16_t);
+  const int tile_slots = pairs / MOE_TILE_ROWS + experts + 1, col_tiles = (n + MOE_TILE_COLS - 1) / MOE_TILE_COLS;
+  if ((long)tile_slots * col_tiles + 8 > 2147483647L) return TS_ERR_SHAPE;
+  const dim3 grid((unsigned)(((tile_slots * col_tiles + 7) / 8) * 8)), block(256);
+  constexpr size_t lds = (size_t)(MOE_TILE_ROWS + MOE_TILE_COLS) * MOE_LDS_ROW * sizeof(uint16_t);
   static_assert(lds <= 80 * 1024, "two workgroups' buffers fit a compute unit's LDS");
   static bool raised = false;  // per process; the attribute belongs to the kernels
   if (!raised) {
@@ -448,8 +456,8 @@ extern "C" int ts_moe_grouped_rows(void* out, const void* in, const void* weight
     raised = true;
   }
   if (gated)
-    hipLaunchKernelGGL(moe_grouped_rows_kernel<true>, grid, block, lds, stream, out, (const bf16_t*)in, (const bf16_t*)weight, order, tile_first, row_first, in_share, n, k, experts, rule);
+    hipLaunchKernelGGL(moe_grouped_rows_kernel<true>, grid, block, lds, stream, out, (const bf16_t*)in, (const bf16_t*)weight, order, tile_first, row_first, in_share, n, k, experts, rule, tile_slots, col_tiles);
   else
-    hipLaunchKernelGGL(moe_grouped_rows_kernel<false>, grid, block, lds, stream, out, (const bf16_t*)in, (const bf16_t*)weight, order, tile_first, row_first, in_share, n, k, experts, rule);
+    hipLaunchKernelGGL(moe_grouped_rows_kernel<false>, grid, block, lds, stream, out, (const bf16_t*)in, (const bf16_t*)weight, order, tile_first, row_first, in_share, n, k, experts, rule, tile_slots, col_tiles);
   return ts_launch_status();
 }
