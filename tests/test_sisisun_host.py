@@ -116,3 +116,13 @@ def test_a_random_model_folder_is_written_and_read_back(tmp_path):
     assert float(tensors["l0.norm1"].abs().max()) == 0.0 and float(tensors["l0.mix.q.norm"].min()) == 1.0
     logits = plain.forward(config, tensors, [5, 1, 96, 40])
     assert logits.shape == (4, 97) and bool(torch.isfinite(logits).all())
+
+
+def test_a_loop_over_no_layers_reads_no_offsets(tmp_path):
+    config = copy.deepcopy(st.CONFIG_Q)
+    config["loop"] = {"start": 1, "stop": 1, "times": 2}
+    _, model = describe_model(config)
+    assert "loop.step" not in model.tensor_specs() and "loop.step" in model.ignorable_names()
+    assert plain.run_order(config) == [(0, None), (1, None)]
+    _, looped = describe_model(st.CONFIG_Q)
+    assert "loop.step" in looped.tensor_specs() and "loop.step" not in looped.ignorable_names()

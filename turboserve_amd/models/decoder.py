@@ -62,6 +62,8 @@ class ModelPlan:
     head: PartSpec
     embedding_prefix: str = "model.embed_tokens"
     head_prefix: str = "lm_head"
+    #: Tensor names a checkpoint of this plan may hold that no part reads.
+    ignorable: tuple[str, ...] = ()
 
     def __post_init__(self) -> None:
         for index, call in enumerate(self.schedule):
@@ -117,7 +119,7 @@ class DecoderModel:
     def ignorable_names(self) -> set[str]:
         """Names a checkpoint may hold that the model does not read (a tied head's own copy of
         the matrix)."""
-        return self.head.ignorable_names()
+        return set(self.head.ignorable_names()) | set(self.plan.ignorable)
 
     def load(self, tensors: Mapping[str, torch.Tensor]) -> None:
         self.embedding.load(tensors)

@@ -70,7 +70,10 @@ def sisisun_plan(config: SisisunConfig) -> ModelPlan:
             enter = PartSpec("pass_offset", {"hidden_size": width, "passes": config.loop_times, "index": entering,
                                              "add_origin": entering > 0})
         schedule.append(LayerCall(index, enter=enter, enter_prefix="loop.step"))
+    # A loop over no layers enters no pass: its table of offsets may be in the file and is not read.
+    unread = () if any(call.enter is not None for call in schedule) else ("loop.step",)
     return ModelPlan(
+        ignorable=unread,
         vocab_size=config.vocab_size,
         hidden_size=width,
         layers=tuple(layers),
