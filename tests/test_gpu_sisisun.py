@@ -465,3 +465,37 @@ def test_greedy_generation_through_the_engine(tmp_path, name):
     # Once more on the same engine: the pages and slots of the first round are used again.
     again = engine.generate(list(reversed(prompts)), SamplingParams(max_tokens=new, temperature=0.0, ignore_eos=True))
     assert [out.new_token_ids for out in again] == list(reversed(want))
+
+
+def test_the_command_line_serves_the_design(tmp_path, capsys):
+    """``engine random-model`` writes a folder from a config.json of the design, ``engine generate``
+    completes prompts given as token ids with the plain implementation's greedy tokens, and
+    ``engine kv-size`` sizes a cache with one group per distinct (heads, key width, value width)."""
+    import re
+
+    from turboserve_amd import cli
+
+    config, _, page = st.TINY["P"]
+    source = tmp_path / "config.json"
+    source.write_text(json.dumps(config))
+    folder = tmp_path / "model"
+    assert cli.main(["engine", "random-model", "--config", str(source), "--out", str(folder), "--seed", "4", "--dtype", "float32"]) == 0
+    raw, tensors = st.read_model_dir(folder)
+    prompts = [st_tokens(config["vocab"], n, 600 + n) for n in (4, 19)]
+    capsys.readouterr()
+    args = ["engine", "generate", "--model", str(folder), "--dtype", "float32", "--max-tokens", "12", "--ignore-eos",
+            "--num-blocks", "24", "--block-size", str(page)]
+    assert cli.main(args + [a for p in prompts for a in ("--prompt-ids", ",".join(map(str, p)))]) == 0
+    shown = [json.loads(m) for m in re.findall(r"^output \d+: (\[.*\])$", capsys.readouterr().out, flags=re.M)]
+    assert len(shown) == len(prompts)
+    for prompt, got in zip(prompts, shown):
+        tokens = list(prompt)
+        for token in got:  # the written model's weights are small: equal logits are allowed for
+            logits = plain.forward(raw, tensors, tokens)[-1]
+            assert float(logits.max() - logits[token]) <= 1e-4 * float(logits.abs().max().clamp_min(1.0))
+            tokens.append(token)
+    assert cli.main(["engine", "kv-size", "--model", str(folder), "--dtype", "bfloat16", "--max-model-len", "64",
+                     "--block-size", str(page)]) == 0
+    sizing = capsys.readouterr().out
+    sizing = json.loads(sizing[sizing.index("{"):])
+    assert len(sizing["num_blocks"]) == 4 and sizing["activation_bytes"] > 0
