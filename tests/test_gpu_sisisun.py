@@ -120,6 +120,25 @@ def test_the_clamped_gated_unit(ops, dtype, inter):
     torch.testing.assert_close(plain_rule, gate.float() * torch.sigmoid(gate.float()) * up.float(), **tol)
 
 
+@pytest.mark.parametrize("rows", [1, 8, 40, 130, 300])
+@pytest.mark.parametrize("rule", [(1.702, 1.5, 1.0), (1.0, 0.0, 0.0)])
+def test_the_gated_unit_applied_by_the_product(ops, rows, rule):
+    """``linear_swiglu`` with a rule: whichever kernel runs the product (the unit in its epilogue,
+    or the product and then the unit's kernel) gives the plain result."""
+    g = torch.Generator().manual_seed(rows)
+    hidden, inter = 256, 192
+    x = torch.randn(rows, hidden, generator=g).to(torch.bfloat16)
+    gate = (0.15 * torch.randn(inter, hidden, generator=g)).to(torch.bfloat16)
+    up = (0.15 * torch.randn(inter, hidden, generator=g)).to(torch.bfloat16)
+    paired = torch.stack([gate, up], dim=1).reshape(2 * inter, hidden).contiguous()
+    got = ops.linear_swiglu(x.to(DEV), paired.to(DEV), rule).float().cpu()
+    gl, ul = x.float() @ gate.float().T, x.float() @ up.float().T
+    if rule[1] > 0:
+        gl, ul = gl.clamp(max=rule[1]), ul.clamp(-rule[1], rule[1])
+    want = gl * torch.sigmoid(rule[0] * gl) * (ul + rule[2])
+    torch.testing.assert_close(got, want, rtol=2e-2, atol=2e-2)
+
+
 @pytest.mark.parametrize("experts, top, groups, keep", [(8, 2, 4, 2), (6, 1, 1, 1), (5, 3, 5, 3), (12, 3, 3, 2), (16, 3, 2, 1),
                                                           (64, 6, 8, 3), (7, 7, 1, 1)])
 def test_the_router_takes_what_the_rule_says(ops, experts, top, groups, keep):

@@ -54,7 +54,7 @@ template <int TN, int MB, int XROWS>
 __global__ void __launch_bounds__(THREADS)
 gemm_tiled_kernel(float* __restrict__ partial, uint16_t* __restrict__ gated, const uint16_t* __restrict__ x,
                   long x_stride, const uint16_t* __restrict__ w, const uint16_t* __restrict__ bias, int m, int n,
-                  int k, int iters_per_split) {
+                  int k, int iters_per_split, GluRule rule) {
   constexpr int NT = 32 * TN;
   static_assert(XROWS == 32 * MB || (XROWS == 16 && MB == 1), "a tile of 32 MB activation rows, or of 16");
   constexpr bool SHARED_ROWS = XROWS == 16;  // both halves of the wavefronts work on the same 16 rows
@@ -179,8 +179,8 @@ gemm_tiled_kernel(float* __restrict__ partial, uint16_t* __restrict__ gated, con
         // bias): the lane holds two such pairs and writes silu(gate) * up for both, rounded once,
         // by the formula of the stand-alone SwiGLU kernel.
         const f32x4 s = acc[a][b];
-        const float lo = s[0] / (1.f + expf(-s[0])) * s[1];
-        const float hi = s[2] / (1.f + expf(-s[2])) * s[3];
+        const float lo = gated_unit(s[0], s[1], rule);
+        const float hi = gated_unit(s[2], s[3], rule);
         uint16_t* out = gated + (size_t)row * (n / 2) + nrow / 2;
         if (nrow + 3 < n) {
           *reinterpret_cast<uint32_t*>(out) =
@@ -205,7 +205,7 @@ gemm_tiled_kernel(float* __restrict__ partial, uint16_t* __restrict__ gated, con
 
 template <int TN, int MB, int XROWS = 32 * MB>
 int launch_tiled_rows(float* partial, uint16_t* gated, const uint16_t* x, long x_stride, const uint16_t* w,
-                      const uint16_t* bias, int m, int n, int k, int iters_per_split, int splits,
+                      const uint16_t* bias, int m, int n, int k, int iters_per_split, int splits, GluRule rule,
                       hipStream_t stream) {
   constexpr int NT = 32 * TN;
   constexpr size_t lds_bytes = (size_t)2 * (NT + XROWS) * LDS_ROW * sizeof(uint16_t);
@@ -221,20 +221,20 @@ int launch_tiled_rows(float* partial, uint16_t* gated, const uint16_t* x, long x
   }
   dim3 grid((n + NT - 1) / NT, splits);
   hipLaunchKernelGGL((gemm_tiled_kernel<TN, MB, XROWS>), grid, dim3(THREADS), lds_bytes, stream, partial, gated, x, x_stride,
-                     w, bias, m, n, k, iters_per_split);
+                     w, bias, m, n, k, iters_per_split, rule);
   return ts_launch_status();
 }
 
 template <int TN>
 int launch_tiled(float* partial, uint16_t* gated, const uint16_t* x, long x_stride, const uint16_t* w,
-                 const uint16_t* bias, int m, int n, int k, int iters_per_split, int splits, hipStream_t stream) {
+                 const uint16_t* bias, int m, int n, int k, int iters_per_split, int splits, GluRule rule, hipStream_t stream) {
   if (m <= 16)
-    return launch_tiled_rows<TN, 1, 16>(partial, gated, x, x_stride, w, bias, m, n, k, iters_per_split, splits, stream);
+    return launch_tiled_rows<TN, 1, 16>(partial, gated, x, x_stride, w, bias, m, n, k, iters_per_split, splits, rule, stream);
   if (m <= 32)
-    return launch_tiled_rows<TN, 1>(partial, gated, x, x_stride, w, bias, m, n, k, iters_per_split, splits, stream);
+    return launch_tiled_rows<TN, 1>(partial, gated, x, x_stride, w, bias, m, n, k, iters_per_split, splits, rule, stream);
   if (m <= 64)
-    return launch_tiled_rows<TN, 2>(partial, gated, x, x_stride, w, bias, m, n, k, iters_per_split, splits, stream);
-  return launch_tiled_rows<TN, 4>(partial, gated, x, x_stride, w, bias, m, n, k, iters_per_split, splits, stream);
+    return launch_tiled_rows<TN, 2>(partial, gated, x, x_stride, w, bias, m, n, k, iters_per_split, splits, rule, stream);
+  return launch_tiled_rows<TN, 4>(partial, gated, x, x_stride, w, bias, m, n, k, iters_per_split, splits, rule, stream);
 }
 
 // Tiles of 256 weight rows (TN = 8): with more than 32 activation rows two buffers no longer fit
@@ -243,11 +243,11 @@ constexpr int M_MAX_TALL = 32;
 
 template <int TN>
 int launch_tiled_tall(float* partial, uint16_t* gated, const uint16_t* x, long x_stride, const uint16_t* w,
-                      const uint16_t* bias, int m, int n, int k, int iters_per_split, int splits, hipStream_t stream) {
+                      const uint16_t* bias, int m, int n, int k, int iters_per_split, int splits, GluRule rule, hipStream_t stream) {
   if (m <= 16)
-    return launch_tiled_rows<TN, 1, 16>(partial, gated, x, x_stride, w, bias, m, n, k, iters_per_split, splits, stream);
+    return launch_tiled_rows<TN, 1, 16>(partial, gated, x, x_stride, w, bias, m, n, k, iters_per_split, splits, rule, stream);
   if (m <= M_MAX_TALL)
-    return launch_tiled_rows<TN, 1>(partial, gated, x, x_stride, w, bias, m, n, k, iters_per_split, splits, stream);
+    return launch_tiled_rows<TN, 1>(partial, gated, x, x_stride, w, bias, m, n, k, iters_per_split, splits, rule, stream);
   return TS_ERR_SHAPE;
 }
 
@@ -259,10 +259,11 @@ int launch_tiled_tall(float* partial, uint16_t* gated, const uint16_t* x, long x
 // tile: 16-row tiles of weights per wavefront, 2, 4 or 5 (a workgroup covers 64, 128 or 160 rows),
 // or, for m <= 32, 8 (256 rows).
 // gated (bfloat16 [m, n / 2], contiguous) instead of partial: w is a gate|up projection whose rows
-// alternate gate, up, and the kernel writes silu(gate) * up; needs splits == 1, no bias, n even.
+// alternate gate, up, and the kernel writes the gated unit of the pair (silu(gate) * up for the rule
+// {1, 0, 0}); needs splits == 1, no bias, n even.
 extern "C" int ts_gemm_tiled(float* partial, void* gated, const void* x, long x_stride, const void* w,
                              const void* bias, int m, int n, int k, int iters_per_split, int splits, int tile,
-                             hipStream_t stream) {
+                             float steepness, float limit, float up_shift, hipStream_t stream) {
   if (m == 0 || n == 0) return TS_OK;
   if (!x || !w || m < 0 || n < 0 || k < 8 || (partial == nullptr) == (gated == nullptr)) return TS_ERR_ARG;
   if (m > M_MAX || (k & 7) != 0 || x_stride < k || (x_stride & 7) != 0) return TS_ERR_SHAPE;
@@ -270,13 +271,14 @@ extern "C" int ts_gemm_tiled(float* partial, void* gated, const void* x, long x_
   if (iters_per_split < 1 || splits != (total + iters_per_split - 1) / iters_per_split || splits > 65535)
     return TS_ERR_SHAPE;
   if (gated && (splits != 1 || bias || (n & 1) != 0)) return TS_ERR_ARG;
+  const GluRule rule = {steepness, limit, up_shift};  // of the gated unit (common.hpp); {1, 0, 0}: silu(gate) * up
   uint16_t* gp = (uint16_t*)gated;
   const uint16_t* xp = (const uint16_t*)x;
   const uint16_t* wp = (const uint16_t*)w;
   const uint16_t* bp = (const uint16_t*)bias;
-  if (tile == 2) return launch_tiled<2>(partial, gp, xp, x_stride, wp, bp, m, n, k, iters_per_split, splits, stream);
-  if (tile == 4) return launch_tiled<4>(partial, gp, xp, x_stride, wp, bp, m, n, k, iters_per_split, splits, stream);
-  if (tile == 5) return launch_tiled<5>(partial, gp, xp, x_stride, wp, bp, m, n, k, iters_per_split, splits, stream);
-  if (tile == 8) return launch_tiled_tall<8>(partial, gp, xp, x_stride, wp, bp, m, n, k, iters_per_split, splits, stream);
+  if (tile == 2) return launch_tiled<2>(partial, gp, xp, x_stride, wp, bp, m, n, k, iters_per_split, splits, rule, stream);
+  if (tile == 4) return launch_tiled<4>(partial, gp, xp, x_stride, wp, bp, m, n, k, iters_per_split, splits, rule, stream);
+  if (tile == 5) return launch_tiled<5>(partial, gp, xp, x_stride, wp, bp, m, n, k, iters_per_split, splits, rule, stream);
+  if (tile == 8) return launch_tiled_tall<8>(partial, gp, xp, x_stride, wp, bp, m, n, k, iters_per_split, splits, rule, stream);
   return TS_ERR_SHAPE;
 }

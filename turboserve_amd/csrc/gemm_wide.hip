@@ -59,7 +59,7 @@ template <int TN, int MB, int WM, int DP, int MODE, bool ONCE>
 __global__ void __launch_bounds__(2 * WM * TS_WAVE)
 gemm_wide_kernel(float* __restrict__ partial, uint16_t* __restrict__ out, const uint16_t* __restrict__ x, long x_stride,
                  const uint16_t* __restrict__ w, const uint16_t* __restrict__ bias, int m, int n, int k,
-                 int iters_per_split, int splits, int n_tiles, int m_tiles) {
+                 int iters_per_split, int splits, int n_tiles, int m_tiles, GluRule rule) {
   typedef WideRegs<TN, MB, WM, DP> Regs;
   constexpr int NT = Regs::NT;
   constexpr int XROWS = Regs::XROWS;
@@ -224,8 +224,8 @@ gemm_wide_kernel(float* __restrict__ partial, uint16_t* __restrict__ out, const 
         // rows of the matrix alternate gate, up: the lane holds two such pairs (the stand-alone
         // SwiGLU kernel's formula, rounded once)
         const f32x4 s = acc[a][b];
-        const float lo = s[0] / (1.f + expf(-s[0])) * s[1];
-        const float hi = s[2] / (1.f + expf(-s[2])) * s[3];
+        const float lo = gated_unit(s[0], s[1], rule);
+        const float hi = gated_unit(s[2], s[3], rule);
         uint16_t* at = out + (size_t)row * (n / 2) + nrow / 2;
         if (nrow + 3 < n) {
           *reinterpret_cast<uint32_t*>(at) =
@@ -263,7 +263,7 @@ gemm_wide_kernel(float* __restrict__ partial, uint16_t* __restrict__ out, const 
 
 template <int TN, int MB, int WM, int DP, int MODE, bool ONCE>
 int launch_wide_kernel(float* partial, uint16_t* out, const uint16_t* x, long x_stride, const uint16_t* w,
-                       const uint16_t* bias, int m, int n, int k, int iters_per_split, int splits, hipStream_t stream) {
+                       const uint16_t* bias, int m, int n, int k, int iters_per_split, int splits, GluRule rule, hipStream_t stream) {
   typedef WideRegs<TN, MB, WM, DP> Regs;
   constexpr size_t lds_bytes = (size_t)2 * (Regs::NT + Regs::XROWS) * Regs::LDS_ROW * sizeof(uint16_t);
   static_assert(lds_bytes <= 160 * 1024, "two buffers must fit the LDS of a compute unit");
@@ -282,21 +282,21 @@ int launch_wide_kernel(float* partial, uint16_t* out, const uint16_t* x, long x_
   const long ids = ((units + DIES - 1) / DIES) * DIES * m_tiles;
   if (ids > 0x7fffffffL) return TS_ERR_SHAPE;
   hipLaunchKernelGGL((gemm_wide_kernel<TN, MB, WM, DP, MODE, ONCE>), dim3((unsigned)ids), dim3(Regs::THREADS), lds_bytes,
-                     stream, partial, out, x, x_stride, w, bias, m, n, k, iters_per_split, splits, n_tiles, m_tiles);
+                     stream, partial, out, x, x_stride, w, bias, m, n, k, iters_per_split, splits, n_tiles, m_tiles, rule);
   return ts_launch_status();
 }
 
 template <int TN, int MB, int WM, int DP>
 int launch_wide(int mode, float* partial, uint16_t* out, const uint16_t* x, long x_stride, const uint16_t* w,
-                const uint16_t* bias, int m, int n, int k, int iters_per_split, int splits, hipStream_t stream) {
+                const uint16_t* bias, int m, int n, int k, int iters_per_split, int splits, GluRule rule, hipStream_t stream) {
   // One tile of activation rows: every weight is read once, with non-temporal loads; more: the
   // tiles over a weight tile share it through their die's L2.
   const bool once = m <= WideRegs<TN, MB, WM, DP>::XROWS;
 #define TS_WIDE_MODE(MODE)                                                                                            \
   return once ? launch_wide_kernel<TN, MB, WM, DP, MODE, true>(partial, out, x, x_stride, w, bias, m, n, k,              \
-                                                           iters_per_split, splits, stream)                           \
+                                                           iters_per_split, splits, rule, stream)                           \
               : launch_wide_kernel<TN, MB, WM, DP, MODE, false>(partial, out, x, x_stride, w, bias, m, n, k,             \
-                                                            iters_per_split, splits, stream)
+                                                            iters_per_split, splits, rule, stream)
   if (mode == 0) TS_WIDE_MODE(0);
   if (mode == 1) TS_WIDE_MODE(1);
   TS_WIDE_MODE(2);
@@ -315,7 +315,7 @@ int launch_wide(int mode, float* partial, uint16_t* out, const uint16_t* x, long
 // wavefronts a workgroup (two, or four, along the activation rows).
 extern "C" int ts_gemm_wide(float* partial, void* out, const void* x, long x_stride, const void* w, const void* bias,
                             int m, int n, int k, int iters_per_split, int splits, int tile, int x_rows, int waves,
-                            int depth, int mode, hipStream_t stream) {
+                            int depth, int mode, float steepness, float limit, float up_shift, hipStream_t stream) {
   if (m == 0 || n == 0) return TS_OK;
   if (!x || !w || m < 0 || n < 0 || k < 8 || mode < 0 || mode > 2) return TS_ERR_ARG;
   if ((mode == 1) != (partial != nullptr) || (mode != 1) != (out != nullptr)) return TS_ERR_ARG;
@@ -325,12 +325,13 @@ extern "C" int ts_gemm_wide(float* partial, void* out, const void* x, long x_str
   if (iters_per_split < 1 || splits != (total + iters_per_split - 1) / iters_per_split) return TS_ERR_SHAPE;
   if (mode != 1 && splits != 1) return TS_ERR_ARG;
   if (mode == 2 && (bias || (n & 1) != 0)) return TS_ERR_ARG;
+  const GluRule rule = {steepness, limit, up_shift};  // of mode 2's gated unit (common.hpp); {1, 0, 0}: silu(gate) * up
   uint16_t* op = (uint16_t*)out;
   const uint16_t* xp = (const uint16_t*)x;
   const uint16_t* wp = (const uint16_t*)w;
   const uint16_t* bp = (const uint16_t*)bias;
 #define TS_WIDE(TN, MB, WM, DP) \
-  return launch_wide<TN, MB, WM, DP>(mode, partial, op, xp, x_stride, wp, bp, m, n, k, iters_per_split, splits, stream)
+  return launch_wide<TN, MB, WM, DP>(mode, partial, op, xp, x_stride, wp, bp, m, n, k, iters_per_split, splits, rule, stream)
   if (depth == 128) {  // tiles of 64 activation rows, eight wavefronts
     if (waves == 8 && x_rows == 64) {
       if (tile == 2) TS_WIDE(2, 1, 4, 128);

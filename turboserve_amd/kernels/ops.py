@@ -70,9 +70,9 @@ _SIGNATURES: dict[str, dict[str, list]] = {
         "ts_gemm_plain": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_long, c_long,
                           c_int, c_int, c_void_p],
         "ts_gemm_tiled": [c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
-                          c_int, c_void_p],
+                          c_int, c_float, c_float, c_float, c_void_p],
         "ts_gemm_wide": [c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
-                         c_int, c_int, c_int, c_int, c_void_p],
+                         c_int, c_int, c_int, c_int, c_float, c_float, c_float, c_void_p],
         "ts_gemm_skinny_resident": [c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
                                     c_int, c_int, c_int, c_void_p],
         "ts_argmax": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
@@ -1094,7 +1094,7 @@ class Ops:
 
     def gemm_tiled(self, x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None,
                    *, max_splits: int | None = None, plan: tuple[int, int, int] | None = None,
-                   gated: bool = False) -> torch.Tensor:
+                   gated: bool = False, rule: tuple[float, float, float] = (1.0, 0.0, 0.0)) -> torch.Tensor:
         """``[S, M, N]`` 32-bit partial sums of ``x [M, K] @ weight [N, K]^T`` over ``S`` ranges of
         K (bias in the first) by the LDS-tiled kernel: M up to 128, K a multiple of 8.  ``plan``
         overrides the grid (iterations per split, splits, tile) for measurements.  ``gated``:
@@ -1115,11 +1115,13 @@ class Ops:
                   "the gated result needs one range of K, no bias and an even number of weight rows")
             out = torch.empty((m, n // 2), dtype=torch.bfloat16, device=x.device)
             _check(self.core.ts_gemm_tiled(None, _ptr(out), _ptr(x), x_stride, _ptr(weight), None, m, n, k,
-                                           per_split, splits, tile, self.stream()), "ts_gemm_tiled")
+                                           per_split, splits, tile, float(rule[0]), float(rule[1]), float(rule[2]), self.stream()),
+                   "ts_gemm_tiled")
             return out
         partial = torch.empty((splits, m, n), dtype=torch.float32, device=x.device)
         _check(self.core.ts_gemm_tiled(_ptr(partial), None, _ptr(x), x_stride, _ptr(weight), _ptr(bias), m, n, k,
-                                       per_split, splits, tile, self.stream()), "ts_gemm_tiled")
+                                       per_split, splits, tile, float(rule[0]), float(rule[1]), float(rule[2]), self.stream()),
+                   "ts_gemm_tiled")
         return partial
 
     #: Up to this many rows a product that was not timed against the BLAS library runs this
@@ -1212,7 +1214,8 @@ class Ops:
         return self.wide_choices[key]
 
     def gemm_wide(self, x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None, *,
-                  plan: tuple[int, int, int, int, int], gated: bool = False, sums: bool = False) -> torch.Tensor:
+                  plan: tuple[int, int, int, int, int], gated: bool = False, sums: bool = False,
+                  rule: tuple[float, float, float] = (1.0, 0.0, 0.0)) -> torch.Tensor:
         """``x [M, K] @ weight [N, K]^T (+ bias)`` by the LDS-tiled kernel for steps of many rows
         (``csrc/gemm_wide.hip``): any M, K a multiple of 8.  ``plan`` = (iterations per range
         of K, ranges, tile, activation rows a workgroup, wavefronts a workgroup[, k per iteration: 64 (the default) or 128]).  One range: bfloat16 ``[M, N]``; several
@@ -1236,16 +1239,17 @@ class Ops:
                   "the gated result needs one range of K, no bias and an even number of weight rows")
             out = self.rows_buffer(m, n // 2, torch.bfloat16, x.device)
             _check(self.core.ts_gemm_wide(None, _ptr(out), _ptr(x), x_stride, _ptr(weight), None, m, n, k, per_split, splits,
-                                          tile, x_rows, waves, depth, 2, self.stream()), "ts_gemm_wide")
+                                          tile, x_rows, waves, depth, 2, float(rule[0]), float(rule[1]), float(rule[2]),
+                                          self.stream()), "ts_gemm_wide")
             return out
         if splits == 1 and not sums:
             out = self.rows_buffer(m, n, torch.bfloat16, x.device)
             _check(self.core.ts_gemm_wide(None, _ptr(out), _ptr(x), x_stride, _ptr(weight), _ptr(bias), m, n, k, per_split,
-                                          splits, tile, x_rows, waves, depth, 0, self.stream()), "ts_gemm_wide")
+                                          splits, tile, x_rows, waves, depth, 0, 1.0, 0.0, 0.0, self.stream()), "ts_gemm_wide")
             return out
         partial = torch.empty((splits, m, n), dtype=torch.float32, device=x.device)
         _check(self.core.ts_gemm_wide(_ptr(partial), None, _ptr(x), x_stride, _ptr(weight), _ptr(bias), m, n, k, per_split,
-                                      splits, tile, x_rows, waves, depth, 1, self.stream()), "ts_gemm_wide")
+                                      splits, tile, x_rows, waves, depth, 1, 1.0, 0.0, 0.0, self.stream()), "ts_gemm_wide")
         return partial
 
     def gemm_resident(self, x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None,
@@ -1435,32 +1439,31 @@ class Ops:
 
     def linear_swiglu(self, x: torch.Tensor, weight: torch.Tensor,
                       rule: tuple[float, float, float] | None = None) -> torch.Tensor:
-        """``silu(gate) * up`` of the projection of ``x`` by a gate|up matrix ``[2 I, K]`` whose rows
-        alternate gate, up -> ``[T, I]`` in the dtype of ``x``.  Decode-sized bfloat16 batches whose
-        product runs as one range of K get the activation in the product's own kernel; every other
-        case is the projection followed by :meth:`swiglu`.  Another gated unit (``rule``, see
-        :meth:`swiglu`) is always the projection followed by the unit's kernel."""
-        if rule is not None and tuple(rule) != (1.0, 0.0, 0.0):
-            return self.swiglu(self.linear(x, weight), x.dtype, paired=True, rule=rule)
+        """The gated unit of the projection of ``x`` by a gate|up matrix ``[2 I, K]`` whose rows
+        alternate gate, up -> ``[T, I]`` in the dtype of ``x``: ``silu(gate) * up``, or another
+        unit by ``rule`` (see :meth:`swiglu`).  bfloat16 products that run as one range of K
+        apply the unit in the product's own kernel; every other case is the projection followed
+        by :meth:`swiglu`."""
+        rule = (1.0, 0.0, 0.0) if rule is None else tuple(float(v) for v in rule)
         if x.dtype == torch.bfloat16 and self.skinny_supported(x, weight) and x.shape[0] <= self.skinny_max_rows:
             _gpu(x, weight)
             if (self._few_rows_wide(x.shape[0], weight.shape[0], weight.shape[1], 1) and weight.shape[0] % 2 == 0
                     and weight.is_contiguous() and x.stride(1) == 1):
                 wide = self._wide_plan_few_rows(x.shape[0], weight.shape[0], weight.shape[1], 1)
-                return self.gemm_wide(x, weight, plan=wide, gated=True)
+                return self.gemm_wide(x, weight, plan=wide, gated=True, rule=rule)
             plan = self._tiled_plan(x.shape[0], weight.shape[0], weight.shape[1], None)
             if plan[1] == 1 and weight.shape[0] % 2 == 0 and weight.is_contiguous() and x.stride(1) == 1:
-                return self.gemm_tiled(x, weight, plan=plan, gated=True)
+                return self.gemm_tiled(x, weight, plan=plan, gated=True, rule=rule)
         elif (x.dtype == torch.bfloat16 and self.skinny_supported_any_rows(x, weight) and weight.shape[0] % 2 == 0
               and weight.is_contiguous() and x.stride(1) == 1):
             _gpu(x, weight)
             m, (n, k) = x.shape[0], weight.shape
             plan = self._wide_plan(m, n, k, True)
-            if self._wide_runs(m, n, k, "gated", plan, lambda: self.gemm_wide(x, weight, plan=plan, gated=True),
-                               lambda: self.swiglu(self._library_product(x, weight, None, None), x.dtype, paired=True)):
-                return self.gemm_wide(x, weight, plan=plan, gated=True)
-            return self.swiglu(self._library_product(x, weight, None, None), x.dtype, paired=True)
-        return self.swiglu(self.linear(x, weight), x.dtype, paired=True)
+            if self._wide_runs(m, n, k, "gated", plan, lambda: self.gemm_wide(x, weight, plan=plan, gated=True, rule=rule),
+                               lambda: self.swiglu(self._library_product(x, weight, None, None), x.dtype, paired=True, rule=rule)):
+                return self.gemm_wide(x, weight, plan=plan, gated=True, rule=rule)
+            return self.swiglu(self._library_product(x, weight, None, None), x.dtype, paired=True, rule=rule)
+        return self.swiglu(self.linear(x, weight), x.dtype, paired=True, rule=rule)
 
     def linear(self, x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None, *,
                for_residual: bool = False) -> torch.Tensor:
