@@ -481,7 +481,7 @@ def test_greedy_generation_through_the_engine(tmp_path, name):
     ))
     outputs = engine.generate(prompts, SamplingParams(max_tokens=new, temperature=0.0, ignore_eos=True))
     assert [out.new_token_ids for out in outputs] == want
-    # Once more on the same engine: the pages and slots of the first round are used again.
+    # Once more on the same engine: the pages and slots of the first run are used again.
     again = engine.generate(list(reversed(prompts)), SamplingParams(max_tokens=new, temperature=0.0, ignore_eos=True))
     assert [out.new_token_ids for out in again] == list(reversed(want))
 

@@ -32,11 +32,13 @@ __device__ __forceinline__ float sum_of_splits(const P* p, int splits, size_t st
   return s;
 }
 
-// One wavefront per (token, q or k head).
+// One wavefront per (token, q or k head) and, with `with_values`, per (token, v head) as well: a
+// step of few tokens then stores its values in the same launch.
 template <typename T, typename P>
 __global__ void __launch_bounds__(64 * HNS_WAVES)
 head_norm_store_kernel(T* q_out, long q_stride, const P* proj, int splits, size_t split_stride,
-                       T* __restrict__ k_pages, const T* __restrict__ q_gain, const T* __restrict__ k_gain,
+                       T* __restrict__ k_pages, T* __restrict__ v_pages, int with_values,
+                       const T* __restrict__ q_gain, const T* __restrict__ k_gain,
                        float eps, float gain_offset, const float* __restrict__ cos_table,
                        const float* __restrict__ sin_table, const int* __restrict__ positions,
                        const int* __restrict__ slots, int tokens, int heads, int kv_heads, int dim, int vdim,
@@ -44,11 +46,26 @@ head_norm_store_kernel(T* q_out, long q_stride, const P* proj, int splits, size_
   __shared__ float held[HNS_WAVES][HNS_MAX_DIM];
   const int wave = threadIdx.x / TS_WAVE, lane = threadIdx.x % TS_WAVE;
   const int qk_heads = heads + kv_heads;
+  const int all_heads = qk_heads + (with_values ? kv_heads : 0);
   const long item = (long)blockIdx.x * HNS_WAVES + wave;
-  const bool active = item < (long)tokens * qk_heads;
-  const int t = active ? (int)(item / qk_heads) : 0;
-  const int h = active ? (int)(item % qk_heads) : 0;
   const size_t width = (size_t)qk_heads * dim + (size_t)kv_heads * vdim;
+  const int item_token = (int)(item / all_heads), item_head = (int)(item % all_heads);
+  const bool is_value = item < (long)tokens * all_heads && item_head >= qk_heads;
+  if (is_value) {
+    // A value head: no norm, no rotation; element d of the token goes to row d of the transposed page.
+    const int slot = slots ? slots[item_token] : -1;
+    if (slot >= 0) {
+      const int kvh = item_head - qk_heads;
+      const P* values = proj + (size_t)item_token * width + (size_t)qk_heads * dim + (size_t)kvh * vdim;
+      T* page = v_pages + ((size_t)(slot / block_size) * kv_heads + kvh) * vdim * block_size + slot % block_size;
+      for (int d = lane; d < vdim; d += TS_WAVE)
+        page[(size_t)d * block_size] = from_float<T>(sum_of_splits(values + d, splits, split_stride));
+    }
+  }
+  // (A value wavefront goes on as an idle one: the barrier below is the whole block's.)
+  const bool active = item < (long)tokens * all_heads && !is_value;
+  const int t = active ? item_token : 0;
+  const int h = active ? item_head : 0;
   const P* row = proj + (size_t)t * width + (size_t)h * dim;
   const T* gain = h < heads ? q_gain : k_gain;
   constexpr int PER_LANE = HNS_MAX_DIM / TS_WAVE;
@@ -207,49 +224,27 @@ value_store_kernel(const P* proj, int splits, size_t split_stride, T* __restrict
   }
 }
 
-// Values of few tokens, or of partial sums: a thread per (token, value dimension), so that the
-// loads of a step of single tokens are all in flight at once.
-template <typename T, typename P>
-__global__ void __launch_bounds__(256)
-value_store_few_kernel(const P* proj, int splits, size_t split_stride, T* __restrict__ v_pages,
-                       const int* __restrict__ slots, int tokens, int heads, int kv_heads, int dim, int vdim,
-                       int block_size) {
-  const int t = blockIdx.x;
-  const int slot = slots[t];
-  if (slot < 0) return;
-  const size_t width = (size_t)(heads + kv_heads) * dim + (size_t)kv_heads * vdim;
-  const P* values = proj + (size_t)t * width + (size_t)(heads + kv_heads) * dim;
-  const size_t page = (size_t)(slot / block_size) * kv_heads;
-  const int offset = slot % block_size;
-  for (int i = threadIdx.x; i < kv_heads * vdim; i += blockDim.x) {
-    const int kvh = i / vdim, d = i % vdim;
-    v_pages[((page + kvh) * vdim + d) * block_size + offset] = from_float<T>(sum_of_splits(values + i, splits, split_stride));
-  }
-}
-
 template <typename T, typename P>
 static void launch_head_norm_store(void* q_out, long q_stride, const void* proj, int splits, long split_stride,
                                    void* k_pages, void* v_pages, const void* q_gain, const void* k_gain, float eps,
                                    float gain_offset, const float* cos_table, const float* sin_table,
                                    const int* positions, const int* slots, int tokens, int heads, int kv_heads,
                                    int dim, int vdim, int block_size, hipStream_t stream) {
-  const long items = (long)tokens * (heads + kv_heads);
+  const bool few = tokens < 4 * HNS_GROUP || splits > 1;  // values in the same launch, a wavefront per value head
+  const long items = (long)tokens * (heads + kv_heads + (few && slots ? kv_heads : 0));
   const bool aligned = ((uintptr_t)q_out | (uintptr_t)proj | (uintptr_t)k_pages | (uintptr_t)q_gain | (uintptr_t)k_gain) % 16 == 0 &&
                        q_stride % 8 == 0 && vdim % 8 == 0;
   if (std::is_same<T, bf16_t>::value && std::is_same<P, bf16_t>::value && splits == 1 && !cos_table && dim % 8 == 0 &&
-      dim <= 128 && tokens >= 4 * HNS_GROUP && aligned)
+      dim <= 128 && !few && aligned)
     hipLaunchKernelGGL(head_norm_store_rows_kernel, dim3((unsigned)((items + 15) / 16)), dim3(256), 0, stream, (bf16_t*)q_out,
                        q_stride, (const bf16_t*)proj, (bf16_t*)k_pages, (const bf16_t*)q_gain, (const bf16_t*)k_gain, eps,
                        gain_offset, slots, tokens, heads, kv_heads, dim, vdim, block_size);
   else
-  hipLaunchKernelGGL((head_norm_store_kernel<T, P>), dim3((unsigned)((items + HNS_WAVES - 1) / HNS_WAVES)),
-                     dim3(64 * HNS_WAVES), 0, stream, (T*)q_out, q_stride, (const P*)proj, splits, (size_t)split_stride,
-                     (T*)k_pages, (const T*)q_gain, (const T*)k_gain, eps, gain_offset, cos_table, sin_table, positions,
-                     slots, tokens, heads, kv_heads, dim, vdim, block_size);
-  if (slots && (tokens < 4 * HNS_GROUP || splits > 1))
-    hipLaunchKernelGGL((value_store_few_kernel<T, P>), dim3(tokens), dim3(256), 0, stream, (const P*)proj, splits,
-                       (size_t)split_stride, (T*)v_pages, slots, tokens, heads, kv_heads, dim, vdim, block_size);
-  else if (slots)
+    hipLaunchKernelGGL((head_norm_store_kernel<T, P>), dim3((unsigned)((items + HNS_WAVES - 1) / HNS_WAVES)),
+                       dim3(64 * HNS_WAVES), 0, stream, (T*)q_out, q_stride, (const P*)proj, splits, (size_t)split_stride,
+                       (T*)k_pages, (T*)v_pages, few && slots ? 1 : 0, (const T*)q_gain, (const T*)k_gain, eps, gain_offset,
+                       cos_table, sin_table, positions, slots, tokens, heads, kv_heads, dim, vdim, block_size);
+  if (slots && !few)
     hipLaunchKernelGGL((value_store_kernel<T, P>), dim3((tokens + HNS_GROUP - 1) / HNS_GROUP, kv_heads), dim3(64), 0,
                        stream, (const P*)proj, splits, (size_t)split_stride, (T*)v_pages, slots, tokens, heads, kv_heads,
                        dim, vdim, block_size);
