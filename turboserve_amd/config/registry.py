@@ -59,3 +59,8 @@ def _ensure_builtin() -> None:
         from turboserve_amd.models.sisisun import sisisun_plan
 
         register_architecture("Sisisun", SisisunConfig.from_dict, sisisun_plan)
+    if "Kisadra" not in ARCHITECTURES:
+        from turboserve_amd.config.kisadra_config import KisadraConfig
+        from turboserve_amd.models.kisadra import kisadra_plan
+
+        register_architecture("Kisadra", KisadraConfig.from_dict, kisadra_plan)

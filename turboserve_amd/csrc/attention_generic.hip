@@ -4,7 +4,11 @@
 // One wavefront per (token, query head).  The token at absolute position p of request s sees
 // the keys lo..p of that request, lo = max(0, p - window + 1) for a windowed layer and 0
 // otherwise (src/turboserve/engine/model/attention.py:139-148: keys <= ctx - q_len + j; the
-// window bound is this engine's).  Keys and values are read through the request's block table
+// window bound is this engine's); with chunk > 0 also lo >= (p / chunk) * chunk: a token sees its
+// own chunk of positions only, chunks counted from position 0 of the request.  sinks > 0 adds that
+// many keys of score 0 without a value to the softmax's denominator.  Without value pages the
+// values are the first vdim elements of the keys themselves (a mixer that caches one vector per
+// token).  Keys and values are read through the request's block table
 // from key pages [NB, Hkv, BS, D] and transposed value pages [NB, Hkv, Dv, BS] (values may be wider
 // or narrower than keys); with softcap c > 0 a scaled score s becomes c * tanh(s / c) before the
 // bias and the softmax; KV head j serves
@@ -27,7 +31,7 @@ paged_attention_generic_kernel(T* __restrict__ out, const T* __restrict__ q, lon
                                const int* __restrict__ block_table, int table_width,
                                const int* __restrict__ token_seq, const int* __restrict__ positions,
                                int heads, int kv_heads, int dim, int vdim, int block_size, float scale,
-                               float softcap, int window, const float* __restrict__ slopes) {
+                               float softcap, int window, const float* __restrict__ slopes, int chunk, float sinks) {
   __shared__ float qs[ATTN_MAX_DIM];
   __shared__ float ps[ATTN_TILE];
   __shared__ long long rows[ATTN_TILE];  // per key of the tile: offset of its value column
@@ -38,7 +42,11 @@ paged_attention_generic_kernel(T* __restrict__ out, const T* __restrict__ q, lon
   const int kvh = h / (heads / kv_heads);
   const int seq = token_seq[t];
   const int p = positions[t];
-  const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+  int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+  if (chunk > 0 && (p / chunk) * chunk > lo) lo = (p / chunk) * chunk;
+  // Values in pages of their own (transposed: a column per key) or inside the key rows.
+  const T* __restrict__ v_src = v_pages ? v_pages : k_pages;
+  const long long v_step = v_pages ? block_size : 1;
   const int* table = block_table + (size_t)seq * table_width;
   // A position encoding may bias the scores by the distance: + slope[h] * (key - p), in 32-bit.
   const float slope = slopes ? slopes[h] : 0.f;
@@ -51,8 +59,9 @@ paged_attention_generic_kernel(T* __restrict__ out, const T* __restrict__ q, lon
   float acc[CHUNKS];
 #pragma unroll
   for (int c = 0; c < CHUNKS; ++c) acc[c] = 0.f;
-  float m_run = -INFINITY;
-  float l_run = 0.f;
+  // A sink is a key of score 0 that is always there: the running maximum starts at its score.
+  float m_run = sinks > 0.f ? 0.f : -INFINITY;
+  float l_run = sinks > 0.f ? sinks : 0.f;
 
   for (int base = lo; base <= p; base += ATTN_TILE) {
     const int key = base + lane;
@@ -62,7 +71,8 @@ paged_attention_generic_kernel(T* __restrict__ out, const T* __restrict__ q, lon
     if (valid) {
       const int blk = table[key / block_size];
       const long long head_base = ((long long)blk * kv_heads + kvh) * block_size * dim;
-      row = ((long long)blk * kv_heads + kvh) * block_size * vdim + (key % block_size);
+      row = v_pages ? ((long long)blk * kv_heads + kvh) * block_size * vdim + (key % block_size)
+                    : head_base + (long long)(key % block_size) * dim;
       const T* krow = k_pages + head_base + (long long)(key % block_size) * dim;
       float s = 0.f;
       for (int d = 0; d < dim; ++d) s = fmaf(qs[d], to_float(krow[d]), s);
@@ -85,7 +95,7 @@ paged_attention_generic_kernel(T* __restrict__ out, const T* __restrict__ q, lon
       if (d < vdim) {
         float a = acc[c] * alpha;
         for (int j = 0; j < count; ++j)
-          a = fmaf(ps[j], to_float(v_pages[rows[j] + (long long)d * block_size]), a);
+          a = fmaf(ps[j], to_float(v_src[rows[j] + (long long)d * v_step]), a);
         acc[c] = a;
       }
     }
@@ -102,24 +112,25 @@ paged_attention_generic_kernel(T* __restrict__ out, const T* __restrict__ q, lon
 
 // out [T, Hq, Dv] contiguous; q rows are q_stride elements apart (the fused projection output).
 // slopes [Hq] (32-bit) or null: the score of key j for the query at position p gets
-// slopes[h] * (j - p) added.
+// slopes[h] * (j - p) added.  v_pages null: the values are the keys' first vdim elements.
 extern "C" int ts_paged_attention_generic(void* out, const void* q, long q_stride,
                                           const void* k_pages, const void* v_pages,
                                           const int* block_table, int table_width,
                                           const int* token_seq, const int* positions, int tokens,
                                           int heads, int kv_heads, int dim, int vdim, int block_size,
-                                          float scale, float softcap, int window, const float* slopes, int dtype,
-                                          hipStream_t stream) {
+                                          float scale, float softcap, int window, const float* slopes, int chunk,
+                                          float sinks, int dtype, hipStream_t stream) {
   if (tokens == 0) return TS_OK;
-  if (!out || !q || !k_pages || !v_pages || !block_table || !token_seq || !positions) return TS_ERR_ARG;
+  if (!out || !q || !k_pages || !block_table || !token_seq || !positions) return TS_ERR_ARG;
+  if (chunk < 0 || !(sinks >= 0.f) || (!v_pages && vdim > dim)) return TS_ERR_ARG;
   if (heads < 1 || kv_heads < 1 || heads % kv_heads != 0 || heads > 65535) return TS_ERR_SHAPE;
   if (dim < 1 || dim > ATTN_MAX_DIM || vdim < 1 || vdim > ATTN_MAX_DIM || block_size < 1 || table_width < 1)
     return TS_ERR_SHAPE;
   dim3 grid(tokens, heads), block(ATTN_TILE);
   if (dtype == TS_F32)
-    hipLaunchKernelGGL(paged_attention_generic_kernel<float>, grid, block, 0, stream, (float*)out, (const float*)q, q_stride, (const float*)k_pages, (const float*)v_pages, block_table, table_width, token_seq, positions, heads, kv_heads, dim, vdim, block_size, scale, softcap, window, slopes);
+    hipLaunchKernelGGL(paged_attention_generic_kernel<float>, grid, block, 0, stream, (float*)out, (const float*)q, q_stride, (const float*)k_pages, (const float*)v_pages, block_table, table_width, token_seq, positions, heads, kv_heads, dim, vdim, block_size, scale, softcap, window, slopes, chunk, sinks);
   else if (dtype == TS_BF16)
-    hipLaunchKernelGGL(paged_attention_generic_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)out, (const bf16_t*)q, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages, block_table, table_width, token_seq, positions, heads, kv_heads, dim, vdim, block_size, scale, softcap, window, slopes);
+    hipLaunchKernelGGL(paged_attention_generic_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)out, (const bf16_t*)q, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages, block_table, table_width, token_seq, positions, heads, kv_heads, dim, vdim, block_size, scale, softcap, window, slopes, chunk, sinks);
   else
     return TS_ERR_DTYPE;
   return ts_launch_status();

@@ -124,12 +124,14 @@ __device__ __forceinline__ ts_u32x4 load_once16(const void* at) {
 }
 
 // The gated unit of a feed-forward: with g' = min(g, limit) and u' = clamp(u, -limit, limit) where
-// limit > 0 (else g' = g, u' = u), g' * sigmoid(steepness * g') * (u' + up_shift).  silu(g) * u is
-// {1, 0, 0}.
+// limit > 0 (else g' = g, u' = u), g' * sigmoid(steepness * (g' + cubic * g'^3)) * (u' + up_shift).
+// silu(g) * u is {1, 0, 0, 0}; the tanh form of GELU, 0.5 g (1 + tanh(c (g + a g^3))), is
+// g * sigmoid(2 c (g + a g^3)): {2 sqrt(2 / pi), 0, 0, 0.044715}.
 struct GluRule {
   float steepness;
   float limit;
   float up_shift;
+  float cubic;
 };
 
 __device__ __forceinline__ float gated_unit(float g, float u, GluRule rule) {
@@ -137,7 +139,8 @@ __device__ __forceinline__ float gated_unit(float g, float u, GluRule rule) {
     g = fminf(g, rule.limit);
     u = fminf(fmaxf(u, -rule.limit), rule.limit);
   }
-  return g / (1.f + expf(-(rule.steepness * g))) * (u + rule.up_shift);
+  const float inner = rule.cubic != 0.f ? fmaf(rule.cubic * g * g, g, g) : g;
+  return g / (1.f + expf(-(rule.steepness * inner))) * (u + rule.up_shift);
 }
 
 static inline int ts_launch_status() { return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH; }

@@ -387,11 +387,11 @@ static void launch_swiglu(void* out, const void* gate_up, int splits, long split
 }
 
 extern "C" int ts_swiglu(void* out, const void* gate_up, int in_f32, int splits, long split_stride,
-                         int tokens, int inter, int paired, float steepness, float limit, float up_shift,
+                         int tokens, int inter, int paired, float steepness, float limit, float up_shift, float cubic,
                          int dtype, hipStream_t stream) {
   if (tokens == 0) return TS_OK;
   if (!out || !gate_up || inter < 1 || splits < 1) return TS_ERR_ARG;
-  const GluRule rule = {steepness, limit, up_shift};
+  const GluRule rule = {steepness, limit, up_shift, cubic};
   if (dtype == TS_F32)
     launch_swiglu<float, float>(out, gate_up, splits, split_stride, tokens, inter, paired, rule, stream);
   else if (dtype == TS_BF16 && in_f32)

@@ -263,7 +263,7 @@ int launch_tiled_tall(float* partial, uint16_t* gated, const uint16_t* x, long x
 // {1, 0, 0}); needs splits == 1, no bias, n even.
 extern "C" int ts_gemm_tiled(float* partial, void* gated, const void* x, long x_stride, const void* w,
                              const void* bias, int m, int n, int k, int iters_per_split, int splits, int tile,
-                             float steepness, float limit, float up_shift, hipStream_t stream) {
+                             float steepness, float limit, float up_shift, float cubic, hipStream_t stream) {
   if (m == 0 || n == 0) return TS_OK;
   if (!x || !w || m < 0 || n < 0 || k < 8 || (partial == nullptr) == (gated == nullptr)) return TS_ERR_ARG;
   if (m > M_MAX || (k & 7) != 0 || x_stride < k || (x_stride & 7) != 0) return TS_ERR_SHAPE;
@@ -271,7 +271,7 @@ extern "C" int ts_gemm_tiled(float* partial, void* gated, const void* x, long x_
   if (iters_per_split < 1 || splits != (total + iters_per_split - 1) / iters_per_split || splits > 65535)
     return TS_ERR_SHAPE;
   if (gated && (splits != 1 || bias || (n & 1) != 0)) return TS_ERR_ARG;
-  const GluRule rule = {steepness, limit, up_shift};  // of the gated unit (common.hpp); {1, 0, 0}: silu(gate) * up
+  const GluRule rule = {steepness, limit, up_shift, cubic};  // of the gated unit (common.hpp); {1, 0, 0}: silu(gate) * up
   uint16_t* gp = (uint16_t*)gated;
   const uint16_t* xp = (const uint16_t*)x;
   const uint16_t* wp = (const uint16_t*)w;

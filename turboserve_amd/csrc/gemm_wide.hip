@@ -315,7 +315,7 @@ int launch_wide(int mode, float* partial, uint16_t* out, const uint16_t* x, long
 // wavefronts a workgroup (two, or four, along the activation rows).
 extern "C" int ts_gemm_wide(float* partial, void* out, const void* x, long x_stride, const void* w, const void* bias,
                             int m, int n, int k, int iters_per_split, int splits, int tile, int x_rows, int waves,
-                            int depth, int mode, float steepness, float limit, float up_shift, hipStream_t stream) {
+                            int depth, int mode, float steepness, float limit, float up_shift, float cubic, hipStream_t stream) {
   if (m == 0 || n == 0) return TS_OK;
   if (!x || !w || m < 0 || n < 0 || k < 8 || mode < 0 || mode > 2) return TS_ERR_ARG;
   if ((mode == 1) != (partial != nullptr) || (mode != 1) != (out != nullptr)) return TS_ERR_ARG;
@@ -325,7 +325,7 @@ extern "C" int ts_gemm_wide(float* partial, void* out, const void* x, long x_str
   if (iters_per_split < 1 || splits != (total + iters_per_split - 1) / iters_per_split) return TS_ERR_SHAPE;
   if (mode != 1 && splits != 1) return TS_ERR_ARG;
   if (mode == 2 && (bias || (n & 1) != 0)) return TS_ERR_ARG;
-  const GluRule rule = {steepness, limit, up_shift};  // of mode 2's gated unit (common.hpp); {1, 0, 0}: silu(gate) * up
+  const GluRule rule = {steepness, limit, up_shift, cubic};  // of mode 2's gated unit (common.hpp); {1, 0, 0}: silu(gate) * up
   uint16_t* op = (uint16_t*)out;
   const uint16_t* xp = (const uint16_t*)x;
   const uint16_t* wp = (const uint16_t*)w;

@@ -2,11 +2,14 @@
 // products for the (token, taken expert) pairs of a step, and the weighted sum.
 //
 // Router: z = R x comes from the engine's own product with a 32-bit result; here, all in 32-bit,
-// s = sigmoid(z).  The experts form `groups` equal groups of
-// neighbours; a group's mark is the sum of its two largest s (its one s if it has one member);
+// s = sigmoid(z), or softmax(z) over all the router's outputs.  Experts are chosen by c = s +
+// correction (a vector per layer; none: c = s).  The experts form `groups` equal groups of
+// neighbours; a group's mark is the sum of its two largest c (its one c if it has one member);
 // only experts of the `keep` groups with the largest marks can be taken; the `top` of them with
-// the largest s are, with weights s / (sum of the taken s + 1e-20) * route_scale.  Equal values go
-// to the lower index.  groups == 1 is plain top-k.
+// the largest c are, with weights s / (sum of the taken s + 1e-20) * route_scale, or, not
+// normalised, s * route_scale.  Equal values go to the lower index.  groups == 1 is plain top-k.
+// An index at or above the number of experts that have matrices stands for the identity (the
+// token itself): the products skip such pairs and the weighted sum reads the token's row.
 #include "common.hpp"
 
 #define MOE_MAX_EXPERTS 1024
@@ -26,14 +29,30 @@ __device__ __forceinline__ int wave_argmax(float value, int index, float& best) 
 __global__ void __launch_bounds__(TS_WAVE)
 moe_select_kernel(int* __restrict__ taken, float* __restrict__ weights, float* __restrict__ extra_gate,
                   const float* __restrict__ z, int stride, int experts, int top, int groups, int keep,
-                  float route_scale) {
-  __shared__ float score[MOE_MAX_EXPERTS];
+                  float route_scale, int softmax, const float* __restrict__ correction, int normalise) {
+  __shared__ float weight_of[MOE_MAX_EXPERTS];  // s: what a taken expert is weighted with
+  __shared__ float score[MOE_MAX_EXPERTS];      // c: what experts are chosen by
   __shared__ float mark[MOE_MAX_EXPERTS];   // per group
   __shared__ int open_group[MOE_MAX_EXPERTS];
   const int t = blockIdx.x;
   const int lane = threadIdx.x;
   const float* row = z + (size_t)t * stride;
-  for (int e = lane; e < experts; e += TS_WAVE) score[e] = 1.f / (1.f + expf(-row[e]));
+  if (softmax) {
+    float top_z = -INFINITY;
+    for (int e = lane; e < experts; e += TS_WAVE) top_z = fmaxf(top_z, row[e]);
+    top_z = wave_max(top_z);
+    float sum = 0.f;
+    for (int e = lane; e < experts; e += TS_WAVE) {
+      const float v = expf(row[e] - top_z);
+      weight_of[e] = v;
+      sum += v;
+    }
+    sum = wave_sum(sum);
+    for (int e = lane; e < experts; e += TS_WAVE) weight_of[e] = weight_of[e] / sum;  // each lane its own entries
+  } else {
+    for (int e = lane; e < experts; e += TS_WAVE) weight_of[e] = 1.f / (1.f + expf(-row[e]));
+  }
+  for (int e = lane; e < experts; e += TS_WAVE) score[e] = weight_of[e] + (correction ? correction[e] : 0.f);
   if (extra_gate && lane == 0) extra_gate[t] = 1.f / (1.f + expf(-row[experts]));
   __syncthreads();
   const int size = experts / groups;
@@ -74,32 +93,36 @@ moe_select_kernel(int* __restrict__ taken, float* __restrict__ weights, float* _
         if (open_group[e / size] && score[e] > mine) { mine = score[e]; at = e; }
       float best;
       const int e = wave_argmax(mine, at, best);
-      if (lane == round) { kept_score = best; kept_index = e; }
-      total += best;
+      const float s = weight_of[e];
+      if (lane == round) { kept_score = s; kept_index = e; }
+      total += s;
       if (lane == 0) score[e] = -INFINITY;  // taken
     }
     __syncthreads();
   }
   if (lane < top) {
     taken[(size_t)t * top + lane] = kept_index;
-    weights[(size_t)t * top + lane] = kept_score / (total + 1e-20f) * route_scale;
+    weights[(size_t)t * top + lane] = (normalise ? kept_score / (total + 1e-20f) : kept_score) * route_scale;
   }
 }
 
 extern "C" int ts_moe_select(int* taken, float* weights, float* extra_gate, const float* z, int tokens, int stride,
-                             int experts, int top, int groups, int keep, float route_scale, hipStream_t stream) {
+                             int experts, int top, int groups, int keep, float route_scale, int softmax,
+                             const float* correction, int normalise, hipStream_t stream) {
   if (tokens == 0) return TS_OK;
   if (!taken || !weights || !z) return TS_ERR_ARG;
   if (experts < 1 || experts > MOE_MAX_EXPERTS || top < 1 || top > MOE_MAX_TOP || groups < 1 || experts % groups != 0 ||
       keep < 1 || keep > groups || top > (experts / groups) * keep || stride < experts + (extra_gate ? 1 : 0))
     return TS_ERR_SHAPE;
   hipLaunchKernelGGL(moe_select_kernel, dim3(tokens), dim3(TS_WAVE), 0, stream, taken, weights, extra_gate, z, stride,
-                     experts, top, groups, keep, route_scale);
+                     experts, top, groups, keep, route_scale, softmax, correction, normalise);
   return ts_launch_status();
 }
 
 // ---------------------------------------------------------------------------------------------
 // The experts' products pair by pair: pair p = (token p / top, its (p % top)-th taken expert e).
+// (Without a list of taken experts, pair p is with expert p mod E: the stacked matrices are then the
+// heads of a per-head product, rows [T * E, K] head by head.)
 // Weights are stacked over the experts, [E, N, K].  out[p, n] = W[e][n] . in[row(p)] with row(p) =
 // p / in_share (the token's activations for the first product: in_share = top; the pair's own row
 // for the second: in_share = 1).  GATED: N = 2 I rows alternate gate, up and the output is
@@ -145,7 +168,7 @@ moe_pair_rows_kernel(void* __restrict__ out_any, const T* __restrict__ in, const
                      const int* __restrict__ taken, int in_share, int n, int k, int experts, GluRule rule) {
   extern __shared__ float xs[];
   const int pair = blockIdx.x;
-  const int e = taken[pair];
+  const int e = taken ? taken[pair] : pair % experts;  // no list: the experts in turn (pair p is with expert p mod E)
   const T* row = in + (size_t)(pair / in_share) * k;
   for (int i = threadIdx.x; i < k; i += blockDim.x) xs[i] = to_float(row[i]);
   __syncthreads();
@@ -173,11 +196,11 @@ moe_pair_rows_kernel(void* __restrict__ out_any, const T* __restrict__ in, const
 
 extern "C" int ts_moe_pair_rows(void* out, const void* in, const void* weight, const int* taken, int pairs,
                                 int in_share, int n, int k, int experts, int gated, float steepness, float limit,
-                                float up_shift, int dtype, hipStream_t stream) {
+                                float up_shift, float cubic, int dtype, hipStream_t stream) {
   if (pairs == 0) return TS_OK;
-  if (!out || !in || !weight || !taken) return TS_ERR_ARG;
+  if (!out || !in || !weight) return TS_ERR_ARG;
   if (n < 1 || k < 1 || k > 12288 || in_share < 1 || experts < 1 || (gated && (n & 1))) return TS_ERR_SHAPE;
-  const GluRule rule = {steepness, limit, up_shift};
+  const GluRule rule = {steepness, limit, up_shift, cubic};
   const int outputs = gated ? n / 2 : n;
   const dim3 grid(pairs, (outputs + MOE_ROWS_PER_BLOCK - 1) / MOE_ROWS_PER_BLOCK), block(256);
   if (grid.y > 65535) return TS_ERR_SHAPE;
@@ -200,16 +223,22 @@ extern "C" int ts_moe_pair_rows(void* out, const void* in, const void* weight, c
 // 32-bit, summed in the order j = 0, 1, ..; `extra` (the shared expert's output) is of type P: T,
 // or `splits` 32-bit partial sums `split_stride` elements apart.
 // ---------------------------------------------------------------------------------------------
-template <typename P>
+// Where `taken` is given, a pair whose index is at or above `experts` is the identity: its output
+// is the token's own row of `rows` (type R), and pair_out holds nothing for it.
+template <typename P, typename R>
 __global__ void moe_combine_kernel(float* __restrict__ out, const float* __restrict__ pair_out,
                                    const float* __restrict__ weights, const P* __restrict__ extra, int splits,
-                                   size_t split_stride, const float* __restrict__ extra_gate, int top, int width) {
+                                   size_t split_stride, const float* __restrict__ extra_gate, int top, int width,
+                                   const int* __restrict__ taken, int experts, const R* __restrict__ rows) {
   const int t = blockIdx.x;
   const int i = blockIdx.y * blockDim.x + threadIdx.x;
   if (i >= width) return;
   float s = 0.f;
-  for (int j = 0; j < top; ++j)
-    s = fmaf(weights[(size_t)t * top + j], pair_out[((size_t)t * top + j) * width + i], s);
+  for (int j = 0; j < top; ++j) {
+    const bool same = taken && taken[(size_t)t * top + j] >= experts;
+    const float y = same ? to_float(rows[(size_t)t * width + i]) : pair_out[((size_t)t * top + j) * width + i];
+    s = fmaf(weights[(size_t)t * top + j], y, s);
+  }
   if (extra) {
     float x = 0.f;
     for (int sp = 0; sp < splits; ++sp) x += to_float(extra[(size_t)sp * split_stride + (size_t)t * width + i]);
@@ -220,17 +249,22 @@ __global__ void moe_combine_kernel(float* __restrict__ out, const float* __restr
 
 extern "C" int ts_moe_combine(float* out, const float* pair_out, const float* weights, const void* extra,
                               int extra_f32, int splits, long split_stride, const float* extra_gate, int tokens,
-                              int top, int width, int dtype, hipStream_t stream) {
+                              int top, int width, int dtype, const int* taken, int experts, const void* rows,
+                              hipStream_t stream) {
   if (tokens == 0) return TS_OK;
   if (!out || !pair_out || !weights || top < 1 || width < 1 || splits < 1) return TS_ERR_ARG;
+  if ((taken != nullptr) != (rows != nullptr)) return TS_ERR_ARG;
   const dim3 grid(tokens, (width + 255) / 256), block(256);
   if (grid.y > 65535) return TS_ERR_SHAPE;
-  if (!extra || extra_f32 || dtype == TS_F32)
-    hipLaunchKernelGGL(moe_combine_kernel<float>, grid, block, 0, stream, out, pair_out, weights, (const float*)extra, splits, (size_t)split_stride, extra_gate, top, width);
-  else if (dtype == TS_BF16)
-    hipLaunchKernelGGL(moe_combine_kernel<bf16_t>, grid, block, 0, stream, out, pair_out, weights, (const bf16_t*)extra, splits, (size_t)split_stride, extra_gate, top, width);
+  if (dtype != TS_F32 && dtype != TS_BF16) return TS_ERR_DTYPE;
+  // `dtype` is the run's: that of `rows`, and of `extra` unless it is 32-bit partial sums.
+  const bool extra32 = !extra || extra_f32 || dtype == TS_F32;
+  if (dtype == TS_F32)
+    hipLaunchKernelGGL((moe_combine_kernel<float, float>), grid, block, 0, stream, out, pair_out, weights, (const float*)extra, splits, (size_t)split_stride, extra_gate, top, width, taken, experts, (const float*)rows);
+  else if (extra32)
+    hipLaunchKernelGGL((moe_combine_kernel<float, bf16_t>), grid, block, 0, stream, out, pair_out, weights, (const float*)extra, splits, (size_t)split_stride, extra_gate, top, width, taken, experts, (const bf16_t*)rows);
   else
-    return TS_ERR_DTYPE;
+    hipLaunchKernelGGL((moe_combine_kernel<bf16_t, bf16_t>), grid, block, 0, stream, out, pair_out, weights, (const bf16_t*)extra, splits, (size_t)split_stride, extra_gate, top, width, taken, experts, (const bf16_t*)rows);
   return ts_launch_status();
 }
 
@@ -259,7 +293,7 @@ moe_group_kernel(int* __restrict__ order, int* __restrict__ tile_first, int* __r
   for (int e = threadIdx.x; e < experts; e += blockDim.x) count[e] = 0;
   __syncthreads();
   for (int p = threadIdx.x; p < pairs; p += blockDim.x) {
-    const int e = taken[p];
+    const int e = taken ? taken[p] : p % experts;
     if (e >= 0 && e < experts) atomicAdd(&count[e], 1);
   }
   __syncthreads();
@@ -277,14 +311,14 @@ moe_group_kernel(int* __restrict__ order, int* __restrict__ tile_first, int* __r
   }
   __syncthreads();
   for (int p = threadIdx.x; p < pairs; p += blockDim.x) {
-    const int e = taken[p];
+    const int e = taken ? taken[p] : p % experts;
     if (e >= 0 && e < experts) order[atomicAdd(&cursor[e], 1)] = p;
   }
 }
 
 extern "C" int ts_moe_group(int* order, int* tile_first, int* row_first, const int* taken, int pairs, int experts,
                             hipStream_t stream) {
-  if (!order || !tile_first || !row_first || !taken || pairs < 1) return TS_ERR_ARG;
+  if (!order || !tile_first || !row_first || pairs < 1) return TS_ERR_ARG;
   if (experts < 1 || experts > MOE_MAX_EXPERTS) return TS_ERR_SHAPE;
   hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(1024), 0, stream, order, tile_first, row_first, taken, pairs, experts);
   return ts_launch_status();
@@ -435,14 +469,14 @@ moe_grouped_rows_kernel(void* __restrict__ out_any, const bf16_t* __restrict__ i
 
 extern "C" int ts_moe_grouped_rows(void* out, const void* in, const void* weight, const int* order,
                                    const int* tile_first, const int* row_first, int pairs, int in_share, int n, int k,
-                                   int experts, int gated, float steepness, float limit, float up_shift,
+                                   int experts, int gated, float steepness, float limit, float up_shift, float cubic,
                                    hipStream_t stream) {
   if (pairs == 0) return TS_OK;
   if (!out || !in || !weight || !order || !tile_first || !row_first) return TS_ERR_ARG;
   if (n < 1 || k < 8 || k % 8 != 0 || in_share < 1 || experts < 1 || experts > MOE_MAX_EXPERTS || (gated && (n & 1)))
     return TS_ERR_SHAPE;
   if (((uintptr_t)in | (uintptr_t)weight) % 16 != 0) return TS_ERR_ARG;
-  const GluRule rule = {steepness, limit, up_shift};
+  const GluRule rule = {steepness, limit, up_shift, cubic};
   const int tile_slots = pairs / MOE_TILE_ROWS + experts + 1, col_tiles = (n + MOE_TILE_COLS - 1) / MOE_TILE_COLS;
   if ((long)tile_slots * col_tiles + 8 > 2147483647L) return TS_ERR_SHAPE;
   const dim3 grid((unsigned)(((tile_slots * col_tiles + 7) / 8) * 8)), block(256);

@@ -34,6 +34,8 @@ MODULES: dict[str, tuple[str, ...]] = {
     "core": (
         "elementwise.hip",
         "head_norm_store.hip",
+        "mixer_store.hip",
+        "linear_state.hip",
         "moe.hip",
         "attention_generic.hip",
         "gemm_plain.hip",

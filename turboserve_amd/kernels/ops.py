@@ -29,6 +29,24 @@ class KernelError(RuntimeError):
     """A kernel refused its arguments or failed to launch."""
 
 
+def glu_rule(rule) -> tuple[float, float, float, float]:
+    """``(steepness, limit, up_shift, cubic)`` of a gated unit ``g' * sigmoid(steepness * (g' + cubic *
+    g'^3)) * (u' + up_shift)`` with ``g' = min(g, limit)``, ``u' = clamp(u, -limit, limit)`` where
+    ``limit > 0``; a rule of three numbers has no cubic term."""
+    values = tuple(float(v) for v in rule)
+    if len(values) == 3:
+        values = (*values, 0.0)
+    if len(values) != 4:
+        raise KernelError(f"a gated unit's rule is (steepness, limit, up_shift[, cubic]), not {rule!r}")
+    return values
+
+
+#: ``silu(gate) * up``.
+SWIGLU_RULE = (1.0, 0.0, 0.0, 0.0)
+#: The tanh form of GELU on the gate: ``0.5 g (1 + tanh(c (g + a g^3))) = g sigmoid(2 c (g + a g^3))``.
+GELU_TANH_RULE = (2.0 * (2.0 / 3.141592653589793) ** 0.5, 0.0, 0.0, 0.044715)
+
+
 def dtype_code(dtype: torch.dtype) -> int:
     if dtype == torch.float32:
         return TS_F32
@@ -43,7 +61,7 @@ _SIGNATURES: dict[str, dict[str, list]] = {
         "ts_rmsnorm": [c_void_p, c_void_p, c_void_p, c_float, c_int, c_int, c_float, c_int, c_int, c_void_p],
         "ts_add_rmsnorm": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_void_p, c_void_p, c_float,
                            c_int, c_int, c_float, c_int, c_int, c_void_p],
-        "ts_swiglu": [c_void_p, c_void_p, c_int, c_int, c_long, c_int, c_int, c_int, c_float, c_float, c_float, c_int,
+        "ts_swiglu": [c_void_p, c_void_p, c_int, c_int, c_long, c_int, c_int, c_int, c_float, c_float, c_float, c_float, c_int,
                       c_void_p],
         "ts_rope_store": [c_void_p, c_long, c_void_p, c_int, c_int, c_long, c_void_p, c_void_p, c_void_p, c_void_p,
                           c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
@@ -51,28 +69,40 @@ _SIGNATURES: dict[str, dict[str, list]] = {
         "ts_patch_tokens": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
         "ts_paged_attention_generic": [c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int,
                                        c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
-                                       c_float, c_float, c_int, c_void_p, c_int, c_void_p],
+                                       c_float, c_float, c_int, c_void_p, c_int, c_float, c_int, c_void_p],
         "ts_head_norm_store": [c_void_p, c_long, c_void_p, c_int, c_int, c_long, c_void_p, c_void_p, c_void_p, c_void_p,
                                c_float, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
                                c_int, c_int, c_int, c_void_p],
+        "ts_span_norm_store": [c_void_p, c_long, c_void_p, c_int, c_int, c_long, c_void_p, c_void_p, c_void_p, c_void_p,
+                               c_float, c_float, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+        "ts_latent_store": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_void_p, c_void_p, c_float, c_void_p,
+                            c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+        "ts_stream_fold": [c_void_p, c_void_p, c_int, c_int, c_long, c_long, c_int, c_int, c_void_p],
+        "ts_stream_pair": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+        "ts_linear_state_scan": [c_void_p, c_void_p, c_int, c_int, c_long, c_void_p, c_void_p, c_float, c_void_p, c_void_p,
+                                 c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
+                                 c_int, c_void_p],
+        "ts_linear_state_carry": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+        "ts_linear_state_finish": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_void_p, c_float, c_int, c_int, c_int,
+                                   c_int, c_int, c_int, c_void_p],
         "ts_embed_positions": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
         "ts_copy_f32": [c_void_p, c_void_p, c_long, c_void_p],
         "ts_stream_offset": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
         "ts_moe_select": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float,
-                          c_void_p],
+                          c_int, c_void_p, c_int, c_void_p],
         "ts_moe_pair_rows": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float,
-                             c_float, c_float, c_int, c_void_p],
+                             c_float, c_float, c_float, c_int, c_void_p],
         "ts_moe_group": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
         "ts_moe_grouped_rows": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
-                                c_int, c_float, c_float, c_float, c_void_p],
+                                c_int, c_float, c_float, c_float, c_float, c_void_p],
         "ts_moe_combine": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_void_p, c_int, c_int, c_int,
-                           c_int, c_void_p],
+                           c_int, c_void_p, c_int, c_void_p, c_void_p],
         "ts_gemm_plain": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_long, c_long,
                           c_int, c_int, c_void_p],
         "ts_gemm_tiled": [c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
-                          c_int, c_float, c_float, c_float, c_void_p],
+                          c_int, c_float, c_float, c_float, c_float, c_void_p],
         "ts_gemm_wide": [c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
-                         c_int, c_int, c_int, c_int, c_float, c_float, c_float, c_void_p],
+                         c_int, c_int, c_int, c_int, c_float, c_float, c_float, c_float, c_void_p],
         "ts_gemm_skinny_resident": [c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
                                     c_int, c_int, c_int, c_void_p],
         "ts_argmax": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
@@ -418,7 +448,7 @@ class Ops:
         inter = width // 2
         out = self.rows_buffer(tokens, inter, out_dtype, gate_up.device)
         _check(self.core.ts_swiglu(_ptr(out), _ptr(gate_up), is_f32, splits, stride, tokens, inter,
-                                   1 if paired else 0, float(rule[0]), float(rule[1]), float(rule[2]),
+                                   1 if paired else 0, *glu_rule(rule),
                                    dtype_code(out_dtype), self.stream()), "ts_swiglu")
         return out
 
@@ -606,18 +636,209 @@ class Ops:
             heads, kv_heads, head_dim, value_dim, block_size, dtype_code(run_dtype), self.stream()), "ts_head_norm_store")
         return q_out, q_stride
 
+    # -- stores and stream steps of other mixers ------------------------------------------------
+
+    def span_norm_store(self, proj: torch.Tensor, k_pages: torch.Tensor | None, v_pages: torch.Tensor | None,
+                        q_gain: torch.Tensor, k_gain: torch.Tensor, eps: float, slots: torch.Tensor | None, tokens: int,
+                        heads: int, kv_heads: int, head_dim: int, value_dim: int, block_size: int,
+                        dtype: torch.dtype | None = None, *, gain_offset: float = 0.0) -> tuple[torch.Tensor, int]:
+        """The store of a mixer whose queries and keys are normalised over their whole projection:
+        of the fused projection ``[T, Hq D + Hkv D + Hkv Dv]`` the ``Hq D`` query elements of a token
+        become ``x * rsqrt(mean(x^2) + eps) * (gain_offset + q_gain)`` (statistics over all heads at
+        once, ``q_gain [Hq D]``), its ``Hkv D`` key elements likewise with ``k_gain [Hkv D]``, in
+        32-bit with one rounding; keys and values go to their pages at ``slots`` (skipped when
+        ``None``).  Returns the tensor that holds the queries and its row stride, as
+        :meth:`rope_store` does."""
+        _gpu(proj, k_pages, v_pages, q_gain, k_gain, slots)
+        _i32(slots, "slots")
+        width = (heads + kv_heads) * head_dim + kv_heads * value_dim
+        run_dtype = dtype or proj.dtype
+        if proj.dim() == 3:
+            _need(dtype is not None, "partial sums need the run dtype")
+        is_f32, splits, stride = self._partials(proj, tokens, width, run_dtype, "projection")
+        _need(q_gain.shape == (heads * head_dim,) and k_gain.shape == (kv_heads * head_dim,) and q_gain.dtype == run_dtype
+              and k_gain.dtype == run_dtype and q_gain.is_contiguous() and k_gain.is_contiguous(),
+              "the gains must be [Hq D] and [Hkv D] of the run dtype")
+        if slots is not None:
+            _need(slots.numel() == tokens, "one slot per token")
+            _need(k_pages is not None and v_pages is not None, "slots need pages")
+            _check_pages(k_pages, v_pages, run_dtype, any_value_width=True)
+            _need(k_pages.shape[1] == kv_heads and k_pages.shape[2] == block_size and k_pages.shape[3] == head_dim
+                  and v_pages.shape[2] == value_dim, "pages do not fit the heads")
+        if is_f32:
+            q_out = self.rows_buffer(tokens, heads * head_dim, run_dtype, proj.device)
+            q_stride = heads * head_dim
+        else:
+            q_out, q_stride = proj, width
+        _check(self.core.ts_span_norm_store(
+            _ptr(q_out), q_stride, _ptr(proj), is_f32, splits, stride, _ptr(k_pages), _ptr(v_pages), _ptr(q_gain),
+            _ptr(k_gain), float(eps), float(gain_offset), _ptr(slots), tokens, heads, kv_heads, head_dim, value_dim,
+            block_size, dtype_code(run_dtype), self.stream()), "ts_span_norm_store")
+        return q_out, q_stride
+
+    def latent_store(self, proj: torch.Tensor, k_pages: torch.Tensor | None, gain: torch.Tensor, eps: float,
+                     cos: torch.Tensor, sin: torch.Tensor, positions: torch.Tensor, slots: torch.Tensor | None,
+                     heads: int, head_dim: int, rot_dim: int, rank: int, block_size: int, max_position: int,
+                     dtype: torch.dtype | None = None) -> tuple[torch.Tensor, torch.Tensor]:
+        """A latent-attention layer's pass over its fused projection ``[T, H (D + R) + C + R]`` (per
+        head ``D`` plain and ``R`` rotated query elements, then the latent of ``C`` and the shared
+        rotated key part of ``R``): the latent is divided by its root mean square and multiplied by
+        ``gain [C]``; of the rotated parts the first ``2 * cos.shape[1]`` elements are turned by the
+        position's angles; ``[latent | rotated key]`` goes to the key pages ``[NB, 1, BS, C + R]`` at
+        ``slots``.  Returns ``(q_plain [T H, D], q_wide [T, H, C + R])``; of ``q_wide`` only the last
+        ``R`` elements of every head are written (the turned query parts)."""
+        _gpu(proj, k_pages, gain, cos, sin, positions, slots)
+        _i32(positions, "positions")
+        _i32(slots, "slots")
+        tokens = positions.numel()
+        width = heads * (head_dim + rot_dim) + rank + rot_dim
+        run_dtype = dtype or proj.dtype
+        if proj.dim() == 3:
+            _need(dtype is not None, "partial sums need the run dtype")
+        is_f32, splits, stride = self._partials(proj, tokens, width, run_dtype, "projection")
+        _need(gain.shape == (rank,) and gain.dtype == run_dtype and gain.is_contiguous(), "the gain must be [C] of the run dtype")
+        _need(cos.shape == sin.shape and cos.dim() == 2 and cos.dtype == torch.float32 and sin.dtype == torch.float32
+              and cos.is_contiguous() and sin.is_contiguous() and 1 <= cos.shape[1] and 2 * cos.shape[1] <= rot_dim,
+              "cos/sin must be float32 [capacity, turned / 2] with turned <= R")
+        _need(max_position < cos.shape[0], f"position {max_position} is beyond the rotary tables ({cos.shape[0]})")
+        if slots is not None:
+            _need(slots.numel() == tokens and k_pages is not None, "one slot per token, and pages")
+            _need(k_pages.dim() == 4 and k_pages.is_contiguous() and k_pages.dtype == run_dtype
+                  and tuple(k_pages.shape[1:]) == (1, block_size, rank + rot_dim), "key pages must be [NB, 1, BS, C + R]")
+        q_plain = torch.empty((tokens * heads, head_dim), dtype=run_dtype, device=proj.device)
+        q_wide = torch.empty((tokens, heads, rank + rot_dim), dtype=run_dtype, device=proj.device)
+        _check(self.core.ts_latent_store(
+            _ptr(q_plain), _ptr(q_wide), _ptr(proj), is_f32, splits, stride, _ptr(k_pages), _ptr(gain), float(eps),
+            _ptr(cos), _ptr(sin), _ptr(positions), _ptr(slots), tokens, heads, head_dim, rot_dim, rank, 2 * cos.shape[1],
+            block_size, dtype_code(run_dtype), self.stream()), "ts_latent_store")
+        return q_plain, q_wide
+
+    def stream_fold(self, residual: torch.Tensor, part: torch.Tensor, dtype: torch.dtype, *, assign: bool = False) -> None:
+        """``residual [T, H] += part`` in 32-bit, in place (``assign``: ``residual = part``); ``part`` is a
+        ``[T, H]`` tensor of the run dtype or ``[S, T, H]`` 32-bit partial sums."""
+        _gpu(residual, part)
+        _need(residual.dim() == 2 and residual.dtype == torch.float32 and residual.is_contiguous(),
+              "residual must be contiguous float32 [T, H]")
+        tokens, hidden = residual.shape
+        is_f32, splits, stride = self._partials(part, tokens, hidden, dtype, "part")
+        _check(self.core.ts_stream_fold(_ptr(residual), _ptr(part), is_f32, splits, stride, tokens * hidden,
+                                        1 if assign else 0, dtype_code(dtype), self.stream()), "ts_stream_fold")
+
+    def stream_pair(self, x: torch.Tensor, origin: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+        """``[T, 2 H]`` of ``dtype``: every row of the 32-bit ``x`` followed by the same row of ``origin``."""
+        _gpu(x, origin)
+        _need(x.dim() == 2 and x.dtype == torch.float32 and x.is_contiguous() and origin.shape == x.shape
+              and origin.dtype == torch.float32 and origin.is_contiguous(), "x and origin must be contiguous float32 [T, H]")
+        tokens, hidden = x.shape
+        out = self.rows_buffer(tokens, 2 * hidden, dtype, x.device)
+        _check(self.core.ts_stream_pair(_ptr(out), _ptr(x), _ptr(origin), tokens, hidden, dtype_code(dtype), self.stream()),
+               "ts_stream_pair")
+        return out
+
+    # -- a state matrix per head instead of cached keys ------------------------------------------
+
+    #: Tokens of a piece when long portions are cut up to run side by side.
+    linear_state_piece = 64
+
+    @staticmethod
+    def linear_state_pieces(query_lens, piece: int) -> tuple[list[list[int]], list[list[int]]]:
+        """For the requests ``0 .. len(query_lens) - 1`` at the front of a step: ``(pieces, carries)``,
+        ``pieces[i] = [request, first row, rows, 0]`` cutting every request's rows into runs of at
+        most ``piece``, ``carries[r] = [request, first piece, pieces, 0]``."""
+        pieces: list[list[int]] = []
+        carries: list[list[int]] = []
+        row = 0
+        for request, count in enumerate(query_lens):
+            carries.append([request, len(pieces), -(-count // piece), 0])
+            for first in range(0, count, piece):
+                pieces.append([request, row + first, min(piece, count - first), 0])
+            row += count
+        return pieces, carries
+
+    def linear_state(self, proj: torch.Tensor, a2: torch.Tensor, a2_bias: torch.Tensor, tau: float, state: torch.Tensor,
+                     state_slots: torch.Tensor, query_start_loc: torch.Tensor, *, tokens: int, first_seq: int,
+                     num_seqs: int, heads: int, head_dim: int, value_dim: int, dtype: torch.dtype,
+                     out: torch.Tensor, plan: tuple | None = None) -> None:
+        """The recurrence ``S <- diag(a_t) S + k_t v_t^T``, ``o_t = S^T q_t`` of a gated-linear-attention
+        layer over the fused projection ``[T, 2 H D + 2 H Dv + R]`` (q, k, v, output gate, the decay's
+        low-rank input ``y``), for the requests ``first_seq .. first_seq + num_seqs - 1`` of the step:
+        ``a_t = sigmoid(a2 y_t + a2_bias)^(1 / tau)`` per key channel, ``q`` scaled by ``D^-0.5``, all
+        in 32-bit; ``state [slots, H, D, Dv]`` 32-bit is read at the requests' ``state_slots`` and left
+        updated; ``o`` goes to the requests' rows of ``out [T, H Dv]`` 32-bit.  Without a ``plan`` each
+        request is walked whole; ``plan = (pieces, carries, n_pieces, n_requests)`` (int32 device
+        tensors from :meth:`linear_state_pieces`, for the requests from 0 on) cuts them into pieces
+        that run side by side."""
+        _gpu(proj, a2, a2_bias, state, state_slots, query_start_loc, out)
+        _i32(state_slots, "state_slots")
+        _i32(query_start_loc, "query_start_loc")
+        low = a2.shape[1]
+        width = 2 * heads * head_dim + 2 * heads * value_dim + low
+        is_f32, splits, stride = self._partials(proj, tokens, width, dtype, "projection")
+        _need(a2.shape == (heads * head_dim, low) and a2.dtype == dtype and a2.is_contiguous()
+              and a2_bias.shape == (heads * head_dim,) and a2_bias.dtype == dtype and a2_bias.is_contiguous(),
+              "a2 [H D, R] and its bias [H D] of the run dtype")
+        _need(head_dim <= 256 and low <= 64, "up to 256 key channels a head and a decay input of up to 64")
+        _need(state.dtype == torch.float32 and state.is_contiguous() and tuple(state.shape[1:]) == (heads, head_dim, value_dim),
+              "state must be contiguous float32 [slots, H, D, Dv]")
+        _need(out.dtype == torch.float32 and out.is_contiguous() and out.shape == (tokens, heads * value_dim),
+              "out must be contiguous float32 [T, H Dv]")
+        _need(query_start_loc.numel() >= first_seq + num_seqs + 1 and state_slots.numel() >= first_seq + num_seqs,
+              "the step's row ranges and state slots do not cover the requests")
+        code = dtype_code(dtype)
+
+        def scan(mode: int, items: int, pieces, piece_state, piece_decay) -> None:
+            _check(self.core.ts_linear_state_scan(
+                _ptr(out), _ptr(proj), is_f32, splits, stride, _ptr(a2), _ptr(a2_bias), float(tau), _ptr(state),
+                _ptr(state_slots), _ptr(query_start_loc), first_seq, _ptr(pieces), _ptr(piece_state), _ptr(piece_decay),
+                items, heads, head_dim, value_dim, low, mode, code, self.stream()), "ts_linear_state_scan")
+
+        if plan is None:
+            scan(0, num_seqs, None, None, None)
+            return
+        pieces, carries, n_pieces, n_requests = plan
+        _need(first_seq == 0 and n_requests == num_seqs, "a plan of pieces covers the requests from the first on")
+        _i32(pieces, "pieces")
+        _i32(carries, "carries")
+        piece_state = torch.empty((n_pieces, heads, head_dim, value_dim), dtype=torch.float32, device=proj.device)
+        piece_decay = torch.empty((n_pieces, heads, head_dim), dtype=torch.float32, device=proj.device)
+        scan(1, n_pieces, pieces, piece_state, piece_decay)
+        _check(self.core.ts_linear_state_carry(_ptr(state), _ptr(state_slots), _ptr(carries), _ptr(piece_state),
+                                               _ptr(piece_decay), n_requests, heads, head_dim, value_dim, self.stream()),
+               "ts_linear_state_carry")
+        scan(2, n_pieces, pieces, piece_state, piece_decay)
+
+    def linear_state_finish(self, o: torch.Tensor, proj: torch.Tensor, gain: torch.Tensor, eps: float, *, heads: int,
+                            head_dim: int, value_dim: int, low: int, dtype: torch.dtype) -> torch.Tensor:
+        """``[T, H Dv]`` of ``dtype``: every head's ``o`` divided by its root mean square (``eps``
+        inside the root), times ``gain [Dv]``, times ``silu`` of the head's output gate, which lies in
+        the projection's rows (see :meth:`linear_state`)."""
+        _gpu(o, proj, gain)
+        tokens = o.shape[0]
+        width = 2 * heads * head_dim + 2 * heads * value_dim + low
+        is_f32, splits, stride = self._partials(proj, tokens, width, dtype, "projection")
+        _need(o.dtype == torch.float32 and o.is_contiguous() and o.shape == (tokens, heads * value_dim), "o must be float32 [T, H Dv]")
+        _need(gain.shape == (value_dim,) and gain.dtype == dtype and gain.is_contiguous(), "gain must be [Dv] of the run dtype")
+        y = self.rows_buffer(tokens, heads * value_dim, dtype, o.device)
+        _check(self.core.ts_linear_state_finish(_ptr(y), _ptr(o), _ptr(proj), is_f32, splits, stride, _ptr(gain), float(eps),
+                                                tokens, heads, head_dim, value_dim, low, dtype_code(dtype), self.stream()),
+               "ts_linear_state_finish")
+        return y
+
     # -- routed feed-forward --------------------------------------------------------------------
 
     def moe_route(self, x: torch.Tensor, router: torch.Tensor, *, top: int, groups: int, keep: int, scale: float,
-                  experts: int | None = None) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor | None]:
+                  experts: int | None = None, softmax: bool = False, correction: torch.Tensor | None = None,
+                  normalise: bool = True) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor | None]:
         """The router of a routed feed-forward: ``z = x router^T`` by the engine's product with a
-        32-bit result, then in 32-bit ``s = sigmoid(z)``; the experts form ``groups`` equal groups
-        of neighbours, a group's mark is the sum of its two largest ``s``, only the ``keep`` best
-        groups' experts can be taken, the ``top`` of them with the largest ``s`` are.  Returns
-        ``(taken [T, top] int32, weights [T, top] float32, gate)``: weights are ``s / (sum of the
-        taken s + 1e-20) * scale``.  With ``experts`` one less than the rows of ``router``, the
-        last row is a gate's vector and ``gate [T]`` the sigmoid of its product (else ``None``)."""
-        _gpu(x, router)
+        32-bit result, then in 32-bit ``s = sigmoid(z)`` or, with ``softmax``, the softmax over the
+        ``experts`` outputs; experts are chosen by ``c = s + correction`` (``correction [experts]``
+        32-bit; none: ``c = s``): they form ``groups`` equal groups of neighbours, a group's mark is
+        the sum of its two largest ``c``, only the ``keep`` best groups' experts can be taken, the
+        ``top`` of them with the largest ``c`` are.  Returns ``(taken [T, top] int32, weights [T, top]
+        float32, gate)``: weights are ``s / (sum of the taken s + 1e-20) * scale``, or ``s * scale``
+        where ``normalise`` is off.  With ``experts`` one less than the rows of ``router``, the last
+        row is a gate's vector and ``gate [T]`` the sigmoid of its product (else ``None``)."""
+        _gpu(x, router, correction)
         _need(x.dim() == 2 and x.is_contiguous() and router.dim() == 2 and router.is_contiguous()
               and router.shape[1] == x.shape[1] and router.dtype == x.dtype, "x [T, H] and router [E, H] of one dtype")
         tokens = x.shape[0]
@@ -625,24 +846,31 @@ class Ops:
         _need(router.shape[0] - experts in (0, 1), "the router holds the experts' rows and at most a gate's")
         _need(1 <= experts <= 1024 and 1 <= top <= 32 and groups >= 1 and experts % groups == 0 and 1 <= keep <= groups
               and top <= (experts // groups) * keep, "a routing rule the kernel does not take")
+        if correction is not None:
+            _need(correction.shape == (experts,) and correction.dtype == torch.float32 and correction.is_contiguous(),
+                  "the correction must be contiguous float32 [experts]")
         z = self.linear_float32_out(x, router)
         _need(z.dtype == torch.float32 and z.stride(1) == 1, "the router's outputs must be 32-bit rows")
         taken = torch.empty((tokens, top), dtype=torch.int32, device=x.device)
         weights = torch.empty((tokens, top), dtype=torch.float32, device=x.device)
         gate = torch.empty((tokens,), dtype=torch.float32, device=x.device) if router.shape[0] > experts else None
         _check(self.core.ts_moe_select(_ptr(taken), _ptr(weights), _ptr(gate), _ptr(z), tokens, z.stride(0), experts, top,
-                                       groups, keep, float(scale), self.stream()), "ts_moe_select")
+                                       groups, keep, float(scale), 1 if softmax else 0, _ptr(correction),
+                                       1 if normalise else 0, self.stream()), "ts_moe_select")
         return taken, weights, gate
 
-    def moe_pair_rows(self, rows: torch.Tensor, weight: torch.Tensor, taken: torch.Tensor, *, share: int,
-                      rule: tuple[float, float, float] | None = None) -> torch.Tensor:
+    def moe_pair_rows(self, rows: torch.Tensor, weight: torch.Tensor, taken: torch.Tensor | None, *, share: int,
+                      rule: tuple[float, float, float] | None = None, pairs: int | None = None) -> torch.Tensor:
         """The product of every (token, taken expert) pair with its expert's matrix out of the
         stack ``weight [E, N, K]``: pair ``p`` (``taken.view(-1)[p]`` its expert) reads row ``p //
         share`` of ``rows [*, K]``.  With ``rule`` the ``N = 2 I`` rows alternate gate, up and the
-        result is the gated unit, ``[P, I]`` of the run dtype; else ``[P, N]`` float32."""
+        result is the gated unit, ``[P, I]`` of the run dtype; else ``[P, N]`` float32.  Without
+        ``taken``, pair ``p`` of ``pairs`` is with expert ``p % E`` (a product per head over rows laid
+        out head by head)."""
         _gpu(rows, weight, taken)
         _i32(taken, "taken")
-        pairs = taken.numel()
+        _need(taken is not None or pairs is not None, "pairs are counted from the taken experts, or given")
+        pairs = taken.numel() if taken is not None else int(pairs)
         _need(weight.dim() == 3 and weight.is_contiguous() and rows.dim() == 2 and rows.is_contiguous()
               and rows.dtype == weight.dtype and rows.shape[1] == weight.shape[2], "rows [*, K] and weight [E, N, K] of one dtype")
         experts, n, k = weight.shape
@@ -654,7 +882,7 @@ class Ops:
             out = torch.empty((pairs, n), dtype=torch.float32, device=rows.device)
         r = rule or (1.0, 0.0, 0.0)
         _check(self.core.ts_moe_pair_rows(_ptr(out), _ptr(rows), _ptr(weight), _ptr(taken), pairs, share, n, k, experts,
-                                          0 if rule is None else 1, float(r[0]), float(r[1]), float(r[2]),
+                                          0 if rule is None else 1, *glu_rule(r),
                                           dtype_code(rows.dtype), self.stream()), "ts_moe_pair_rows")
         return out
 
@@ -662,22 +890,39 @@ class Ops:
     #: matrix cores (below it every pair streams its expert's matrices, which is what few tokens cost anyway).
     moe_grouped_min_tokens = 33
 
-    def moe_grouping(self, taken: torch.Tensor, experts: int, dtype: torch.dtype, *widths: int):
+    def moe_grouping(self, taken: torch.Tensor | None, experts: int, dtype: torch.dtype, *widths: int,
+                     pairs: int | None = None):
         """``(order, tile_first, row_first)`` for :meth:`moe_grouped_rows` where a step's pairs are
         worth grouping by expert (bfloat16, many tokens, every inner width a multiple of 8), else
-        ``None``.  All on the device: the host never sees who took which expert."""
+        ``None``.  All on the device: the host never sees who took which expert.  Without ``taken``,
+        pair ``p`` of ``pairs`` is with expert ``p % experts``."""
         _gpu(taken)
         _i32(taken, "taken")
-        if (dtype != torch.bfloat16 or taken.shape[0] < self.moe_grouped_min_tokens or experts > 1024
+        tokens = taken.shape[0] if taken is not None else int(pairs) // experts
+        if (dtype != torch.bfloat16 or tokens < self.moe_grouped_min_tokens or experts > 1024
                 or any(w % 8 != 0 for w in widths)):
             return None
-        pairs = taken.numel()
-        order = torch.empty((pairs,), dtype=torch.int32, device=taken.device)
-        tile_first = torch.empty((experts + 1,), dtype=torch.int32, device=taken.device)
-        row_first = torch.empty((experts + 1,), dtype=torch.int32, device=taken.device)
+        pairs = taken.numel() if taken is not None else int(pairs)
+        device = taken.device if taken is not None else self.device
+        order = torch.empty((pairs,), dtype=torch.int32, device=device)
+        tile_first = torch.empty((experts + 1,), dtype=torch.int32, device=device)
+        row_first = torch.empty((experts + 1,), dtype=torch.int32, device=device)
         _check(self.core.ts_moe_group(_ptr(order), _ptr(tile_first), _ptr(row_first), _ptr(taken), pairs, experts,
                                       self.stream()), "ts_moe_group")
         return order, tile_first, row_first
+
+    def per_head_rows(self, rows: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+        """``[T H, N]`` float32: row ``t H + h`` of ``rows [T H, K]`` against head ``h``'s matrix of the
+        stack ``weight [H, N, K]``.  The heads are the experts of a routed product that every token
+        takes in turn, so the same kernels run it: head by head for few tokens, grouped through the
+        matrix cores for many."""
+        heads, n, k = weight.shape
+        pairs = rows.shape[0]
+        _need(pairs % heads == 0, "rows are laid out head by head")
+        grouping = self.moe_grouping(None, heads, rows.dtype, k, pairs=pairs)
+        if grouping is not None:
+            return self.moe_grouped_rows(rows, weight, grouping, pairs, share=1)
+        return self.moe_pair_rows(rows, weight, None, share=1, pairs=pairs)
 
     def moe_grouped_rows(self, rows: torch.Tensor, weight: torch.Tensor, grouping: tuple, pairs: int, *, share: int,
                          rule: tuple[float, float, float] | None = None) -> torch.Tensor:
@@ -699,7 +944,7 @@ class Ops:
         r = rule or (1.0, 0.0, 0.0)
         _check(self.core.ts_moe_grouped_rows(_ptr(out), _ptr(rows), _ptr(weight), _ptr(order), _ptr(tile_first),
                                              _ptr(row_first), pairs, share, n, k, experts, 0 if rule is None else 1,
-                                             float(r[0]), float(r[1]), float(r[2]), self.stream()), "ts_moe_grouped_rows")
+                                             *glu_rule(r), self.stream()), "ts_moe_grouped_rows")
         return out
 
     def moe_expert_units(self, x: torch.Tensor, gate_up: torch.Tensor, taken: torch.Tensor,
@@ -718,11 +963,15 @@ class Ops:
         return self.moe_pair_rows(units, down, taken, share=1)
 
     def moe_combine(self, pair_out: torch.Tensor, weights: torch.Tensor, extra: torch.Tensor | None = None,
-                    extra_gate: torch.Tensor | None = None, dtype: torch.dtype | None = None) -> torch.Tensor:
+                    extra_gate: torch.Tensor | None = None, dtype: torch.dtype | None = None, *,
+                    taken: torch.Tensor | None = None, experts: int = 0, rows: torch.Tensor | None = None) -> torch.Tensor:
         """``[1, T, H]`` float32 (one partial sum for the residual stream): the pairs' outputs
         ``[T * top, H]`` weighted by ``weights [T, top]`` and summed per token, plus ``extra_gate [T]``
-        times ``extra`` (``[T, H]`` of ``dtype`` or ``[S, T, H]`` 32-bit partial sums) where given."""
-        _gpu(pair_out, weights, extra, extra_gate)
+        times ``extra`` (``[T, H]`` of ``dtype`` or ``[S, T, H]`` 32-bit partial sums) where given.
+        With ``taken [T, top]``, ``experts`` and ``rows [T, H]`` (the feed-forward's input), a pair
+        whose index is ``>= experts`` is the identity: it contributes its token's row of ``rows``,
+        and its row of ``pair_out`` is not read."""
+        _gpu(pair_out, weights, extra, extra_gate, taken, rows)
         tokens, top = weights.shape
         _need(pair_out.dtype == torch.float32 and pair_out.is_contiguous() and pair_out.dim() == 2
               and pair_out.shape[0] == tokens * top and weights.dtype == torch.float32 and weights.is_contiguous(),
@@ -735,9 +984,17 @@ class Ops:
             code = dtype_code(run)
         if extra_gate is not None:
             _need(extra_gate.shape == (tokens,) and extra_gate.dtype == torch.float32, "extra_gate must be float32 [T]")
+        _need((taken is None) == (rows is None), "identity pairs need both the taken experts and the input rows")
+        if taken is not None:
+            _i32(taken, "taken")
+            _need(taken.shape == (tokens, top) and rows.shape == (tokens, hidden) and rows.is_contiguous(),
+                  "taken [T, top] and rows [T, H]")
+            _need(extra is None or is_f32 or rows.dtype == (dtype or extra.dtype), "rows and extra must share the run dtype")
+            code = dtype_code(rows.dtype)
         out = torch.empty((1, tokens, hidden), dtype=torch.float32, device=pair_out.device)
         _check(self.core.ts_moe_combine(_ptr(out), _ptr(pair_out), _ptr(weights), _ptr(extra), is_f32, splits, stride,
-                                        _ptr(extra_gate), tokens, top, hidden, code, self.stream()), "ts_moe_combine")
+                                        _ptr(extra_gate), tokens, top, hidden, code, _ptr(taken), int(experts), _ptr(rows),
+                                        self.stream()), "ts_moe_combine")
         return out
 
     # -- attention ----------------------------------------------------------------------------
@@ -747,7 +1004,7 @@ class Ops:
         q: torch.Tensor,
         q_stride: int,
         k_pages: torch.Tensor,
-        v_pages: torch.Tensor,
+        v_pages: torch.Tensor | None,
         block_table: torch.Tensor,
         token_seq: torch.Tensor,
         positions: torch.Tensor,
@@ -756,6 +1013,10 @@ class Ops:
         window: int | None,
         slopes: torch.Tensor | None = None,
         softcap: float = 0.0,
+        *,
+        chunk: int | None = None,
+        sinks: float = 0.0,
+        value_dim: int | None = None,
     ) -> torch.Tensor:
         """Attention of every token over the keys ``lo..position`` of its request.  With
         ``softcap = c > 0`` a scaled score ``s`` becomes ``c * tanh(s / c)``.  Values may have a
@@ -763,8 +1024,10 @@ class Ops:
 
         ``q`` is the tensor whose first ``heads * D`` elements of each ``q_stride``-long row
         are the (already encoded) queries.  ``slopes [heads]`` (32-bit), if given, biases the
-        score of key ``j`` for a query at position ``p`` by ``slopes[h] * (j - p)``.  Returns
-        ``[T, heads * D]``."""
+        score of key ``j`` for a query at position ``p`` by ``slopes[h] * (j - p)``.  ``chunk = C``:
+        a query at ``p`` sees no key below ``(p // C) * C``.  ``sinks = n``: the softmax's denominator
+        counts ``n`` more keys of score 0 that have no value.  ``v_pages = None`` with ``value_dim =
+        Dv <= D``: a key's value is its own first ``Dv`` elements."""
         _gpu(q, k_pages, v_pages, block_table, token_seq, positions)
         if slopes is not None:
             _gpu(slopes)
@@ -773,10 +1036,17 @@ class Ops:
         _i32(block_table, "block_table")
         _i32(token_seq, "token_seq")
         _i32(positions, "positions")
-        _check_pages(k_pages, v_pages, q.dtype, any_value_width=True)
+        if v_pages is not None:
+            _check_pages(k_pages, v_pages, q.dtype, any_value_width=True)
+            value_dim = v_pages.shape[2]
+        else:
+            _need(k_pages.dim() == 4 and k_pages.is_contiguous() and k_pages.dtype == q.dtype,
+                  "key pages must be a contiguous [NB, Hkv, BS, D] tensor of the queries' dtype")
+            _need(value_dim is not None and 1 <= value_dim <= k_pages.shape[3],
+                  "values inside the keys are their first value_dim elements")
         _, kv_heads, block_size, head_dim = k_pages.shape
-        value_dim = v_pages.shape[2]
         _need(value_dim <= ATTENTION_MAX_HEAD_DIM, f"values of {value_dim} elements are wider than the kernel takes")
+        _need((chunk is None or chunk >= 1) and sinks >= 0.0, "a chunk is at least one position, sinks are not negative")
         tokens = positions.numel()
         _need(q.is_contiguous() and q.numel() >= tokens * q_stride and q_stride >= heads * head_dim,
               "q does not hold [T, q_stride] rows")
@@ -788,7 +1058,7 @@ class Ops:
             _ptr(out), _ptr(q), q_stride, _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
             block_table.shape[1], _ptr(token_seq), _ptr(positions), tokens, heads, kv_heads, head_dim, value_dim,
             block_size, float(scale), float(softcap), int(window or 0), _ptr(slopes) if slopes is not None else None,
-            dtype_code(q.dtype), self.stream()),
+            int(chunk or 0), float(sinks), dtype_code(q.dtype), self.stream()),
             "ts_paged_attention_generic")
         return out
 
@@ -1115,12 +1385,12 @@ class Ops:
                   "the gated result needs one range of K, no bias and an even number of weight rows")
             out = torch.empty((m, n // 2), dtype=torch.bfloat16, device=x.device)
             _check(self.core.ts_gemm_tiled(None, _ptr(out), _ptr(x), x_stride, _ptr(weight), None, m, n, k,
-                                           per_split, splits, tile, float(rule[0]), float(rule[1]), float(rule[2]), self.stream()),
+                                           per_split, splits, tile, *glu_rule(rule), self.stream()),
                    "ts_gemm_tiled")
             return out
         partial = torch.empty((splits, m, n), dtype=torch.float32, device=x.device)
         _check(self.core.ts_gemm_tiled(_ptr(partial), None, _ptr(x), x_stride, _ptr(weight), _ptr(bias), m, n, k,
-                                       per_split, splits, tile, float(rule[0]), float(rule[1]), float(rule[2]), self.stream()),
+                                       per_split, splits, tile, *glu_rule(rule), self.stream()),
                    "ts_gemm_tiled")
         return partial
 
@@ -1239,17 +1509,17 @@ class Ops:
                   "the gated result needs one range of K, no bias and an even number of weight rows")
             out = self.rows_buffer(m, n // 2, torch.bfloat16, x.device)
             _check(self.core.ts_gemm_wide(None, _ptr(out), _ptr(x), x_stride, _ptr(weight), None, m, n, k, per_split, splits,
-                                          tile, x_rows, waves, depth, 2, float(rule[0]), float(rule[1]), float(rule[2]),
+                                          tile, x_rows, waves, depth, 2, *glu_rule(rule),
                                           self.stream()), "ts_gemm_wide")
             return out
         if splits == 1 and not sums:
             out = self.rows_buffer(m, n, torch.bfloat16, x.device)
             _check(self.core.ts_gemm_wide(None, _ptr(out), _ptr(x), x_stride, _ptr(weight), _ptr(bias), m, n, k, per_split,
-                                          splits, tile, x_rows, waves, depth, 0, 1.0, 0.0, 0.0, self.stream()), "ts_gemm_wide")
+                                          splits, tile, x_rows, waves, depth, 0, 1.0, 0.0, 0.0, 0.0, self.stream()), "ts_gemm_wide")
             return out
         partial = torch.empty((splits, m, n), dtype=torch.float32, device=x.device)
         _check(self.core.ts_gemm_wide(_ptr(partial), None, _ptr(x), x_stride, _ptr(weight), _ptr(bias), m, n, k, per_split,
-                                      splits, tile, x_rows, waves, depth, 1, 1.0, 0.0, 0.0, self.stream()), "ts_gemm_wide")
+                                      splits, tile, x_rows, waves, depth, 1, 1.0, 0.0, 0.0, 0.0, self.stream()), "ts_gemm_wide")
         return partial
 
     def gemm_resident(self, x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None,

@@ -27,7 +27,13 @@ class GroupedQueryAttention(Mixer):
     ``head_norm = {"eps": e, "gain_offset": o}`` (every q and k head is divided by its root mean
     square, eps inside the root, and multiplied by ``o +`` a gain vector ``[D]`` that all heads
     share, one for q and one for k, in 32-bit, before the position encoding); ``softcap = c``
-    (a scaled score ``s`` becomes ``c * tanh(s / c)`` before the softmax).  ``names``: the tensor
+    (a scaled score ``s`` becomes ``c * tanh(s / c)`` before the softmax); ``span_norm = {"eps": e,
+    "gain_offset": o}`` (all q heads of a token together are divided by their root mean square and
+    multiplied by ``o +`` a gain of their full size ``[Hq D]``, the k heads likewise with a gain ``[Hkv
+    D]``, stored under the same names as the per-head gains); ``chunk = C`` (the token at position
+    ``i`` sees only keys from ``(i // C) * C`` on: chunks of positions counted from the request's
+    start); ``sinks = n`` (the softmax's denominator counts ``n`` more keys of score 0 that have no
+    value).  ``names``: the tensor
     names under the part's prefix of ``q, k, v, o`` (biases: the same with ``weight`` replaced by
     ``bias``) and of the two gains."""
 
@@ -49,6 +55,9 @@ class GroupedQueryAttention(Mixer):
         head_norm: Mapping | None = None,
         softcap: float = 0.0,
         names: Mapping[str, str] | None = None,
+        span_norm: Mapping | None = None,
+        chunk: int | None = None,
+        sinks: float = 0.0,
     ) -> None:
         super().__init__(prefix, runtime)
         # Refused here, when the model is put together, not at the first step after the weights
@@ -71,6 +80,16 @@ class GroupedQueryAttention(Mixer):
         self.softcap = float(softcap)
         self.head_norm_eps = None if head_norm is None else float(head_norm["eps"])
         self.head_norm_offset = 0.0 if head_norm is None else float(head_norm.get("gain_offset", 0.0))
+        if span_norm is not None and head_norm is not None:
+            raise ValueError(f"{prefix or 'attention'}: a norm per head and one over the whole projection exclude each other")
+        self.span_norm_eps = None if span_norm is None else float(span_norm["eps"])
+        self.span_norm_offset = 0.0 if span_norm is None else float(span_norm.get("gain_offset", 0.0))
+        self.chunk = None if chunk is None else int(chunk)
+        if self.chunk is not None and self.chunk < 1:
+            raise ValueError(f"{prefix or 'attention'}: a chunk of {self.chunk} positions")
+        self.sinks = float(sinks)
+        if self.sinks < 0:
+            raise ValueError(f"{prefix or 'attention'}: {self.sinks} sinks")
         self.names = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight",
                       "q_norm": "q_norm.weight", "k_norm": "k_norm.weight", **(names or {})}
         self.q_size = self.num_heads * self.head_dim
@@ -116,6 +135,10 @@ class GroupedQueryAttention(Mixer):
             init = "zeros" if self.head_norm_offset == 1.0 else "ones"
             specs[self.name(self.names["q_norm"])] = TensorSpec((self.head_dim,), init=init)
             specs[self.name(self.names["k_norm"])] = TensorSpec((self.head_dim,), init=init)
+        if self.span_norm_eps is not None:
+            init = "zeros" if self.span_norm_offset == 1.0 else "ones"
+            specs[self.name(self.names["q_norm"])] = TensorSpec((self.q_size,), init=init)
+            specs[self.name(self.names["k_norm"])] = TensorSpec((self.kv_size,), init=init)
         specs.update(self.position.tensor_specs())
         return specs
 
@@ -136,7 +159,7 @@ class GroupedQueryAttention(Mixer):
         self.o_weight = tensors[self.name(self.names["o"])].contiguous()
         if self.out_bias:
             self.o_bias_tensor = tensors[self.name(self._bias("o"))].contiguous()
-        if self.head_norm_eps is not None:
+        if self.head_norm_eps is not None or self.span_norm_eps is not None:
             self.q_gain = tensors[self.name(self.names["q_norm"])].contiguous()
             self.k_gain = tensors[self.name(self.names["k_norm"])].contiguous()
         self.position.load(tensors)
@@ -149,6 +172,8 @@ class GroupedQueryAttention(Mixer):
             more["value_dim"] = self.value_dim
         if self.head_norm_eps is not None:
             more["head_norm"] = (self.q_gain, self.k_gain, self.head_norm_eps, self.head_norm_offset)
+        if self.span_norm_eps is not None:
+            more["span_norm"] = (self.q_gain, self.k_gain, self.span_norm_eps, self.span_norm_offset)
         q, q_stride = self.position.encode_and_store(
             qkv, self.num_heads, self.num_kv_heads, self.head_dim, ctx, cache, **more
         )
@@ -166,7 +191,7 @@ class GroupedQueryAttention(Mixer):
         ops = self.runtime.ops
         table = ctx.block_tables[cache.group]
         slopes = self.position.score_slopes(self.num_heads)
-        fast = (slopes is None and self.value_dim == self.head_dim
+        fast = (slopes is None and self.value_dim == self.head_dim and self.chunk is None and self.sinks == 0.0
                 and ops.mfma_attention_supported(qkv.dtype, self.head_dim, cache.block_size))
         if fast:
             out = ops.rows_buffer(ctx.num_tokens, self.out_size, qkv.dtype, qkv.device)
@@ -192,5 +217,5 @@ class GroupedQueryAttention(Mixer):
             return out
         return ops.paged_attention_generic(
             qkv, q_stride, cache.k, cache.v, table, ctx.token_seq, ctx.positions,
-            self.num_heads, self.scale, self.window, slopes, self.softcap,
+            self.num_heads, self.scale, self.window, slopes, self.softcap, chunk=self.chunk, sinks=self.sinks,
         )

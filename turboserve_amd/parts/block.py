@@ -74,3 +74,61 @@ class PreNormBlock(Block):
         x = self.ff_norm.forward_residual(stream)
         stream.pending = self.feed_forward.forward(x, ctx)
         return stream
+
+
+@register_block("parallel")
+class ParallelBlock(Block):
+    """``h += mixer(n) + feed_forward(n)`` with one ``n = norm(h)`` that both parts read.
+
+    The mixer's output is added into the 32-bit residual stream by a pass of its own
+    (``ops.stream_fold``); the feed-forward's waits in ``stream.pending`` for the next norm, as in
+    the pre-norm block.  A block without a feed-forward (``feed_forward=None``) leaves the mixer's
+    output pending instead.  ``norm_name`` / ``mixer_name`` / ``ff_name`` are the checkpoint names
+    of the parts under the block's prefix."""
+
+    def __init__(
+        self,
+        prefix: str,
+        runtime: Runtime,
+        *,
+        mixer: PartSpec,
+        feed_forward: PartSpec | None,
+        norm: PartSpec,
+        mixer_name: str = "mix",
+        ff_name: str = "mlp",
+        norm_name: str = "norm1",
+    ) -> None:
+        super().__init__(prefix, runtime)
+        self.norm = build_part("norm", norm, self.name(norm_name), runtime)
+        self.mixer = build_part("mixer", mixer, self.name(mixer_name), runtime)
+        self.feed_forward = None
+        if feed_forward is not None:
+            self.feed_forward = build_part("feed_forward", feed_forward, self.name(ff_name), runtime)
+
+    def parts(self) -> list[Part]:
+        return [self.norm, self.mixer] if self.feed_forward is None else [self.norm, self.mixer, self.feed_forward]
+
+    def activation_bytes(self, tokens: int, itemsize: int) -> int:
+        """The norm's output stays alive while both parts run, one after the other."""
+        largest = max(part.activation_bytes(tokens, itemsize) for part in self.parts()[1:])
+        return self.norm.activation_bytes(tokens, itemsize) + largest
+
+    def tensor_specs(self) -> dict[str, TensorSpec]:
+        specs: dict[str, TensorSpec] = {}
+        for part in self.parts():
+            specs.update(part.tensor_specs())
+        return specs
+
+    def load(self, tensors: Mapping[str, torch.Tensor]) -> None:
+        for part in self.parts():
+            part.load(tensors)
+
+    def forward(self, stream: ResidualStream, ctx, cache: CacheView) -> ResidualStream:
+        x = self.norm.forward_residual(stream)
+        mixed = self.mixer.forward(x, ctx, cache)
+        if self.feed_forward is None:
+            stream.pending = mixed
+            return stream
+        self.runtime.ops.stream_fold(stream.residual, mixed, self.runtime.dtype)
+        stream.pending = self.feed_forward.forward(x, ctx)
+        return stream

@@ -24,6 +24,13 @@ class RoutedExperts(FeedForward):
     token runs through, under ``<prefix>.<shared_name>``; with ``shared_gate_name`` its output
     is multiplied by ``sigmoid(v . x)``, one number per token, ``v`` the tensor of that name.
 
+    Other routers, each a parameter: ``router_scores = "softmax"`` (``s`` is the softmax over all the
+    router's outputs); ``correction_name`` (a vector ``[outputs]`` under the part's prefix that is
+    added to ``s`` where experts are chosen, while the weights use ``s`` alone); ``normalise =
+    False`` (weights ``s * route_scale``, not divided by their sum); ``identity = n`` (the router
+    has ``experts + n`` outputs, and the last ``n`` stand for the token itself: such a pair
+    contributes ``w * x`` and has no matrices).
+
     The experts' matrices are stacked at load: ``[E, 2 I, H]`` with rows alternating gate, up,
     and ``[E, H, I]``.  A step routes on the device, runs every (token, taken expert) pair
     against its expert's matrices (pair by pair in steps of few tokens, grouped by expert on the
@@ -49,6 +56,10 @@ class RoutedExperts(FeedForward):
         shared_gate_name: str | None = None,
         router_name: str = "router",
         expert_names: tuple[str, str, str, str] = ("e{index}", "gate", "up", "down"),
+        router_scores: str = "sigmoid",
+        correction_name: str | None = None,
+        normalise: bool = True,
+        identity: int = 0,
     ) -> None:
         super().__init__(prefix, runtime)
         self.hidden_size = int(hidden_size)
@@ -59,14 +70,25 @@ class RoutedExperts(FeedForward):
         self.keep = int(keep)
         self.route_scale = float(route_scale)
         self.rule = tuple(float(v) for v in rule)
-        if self.experts < 1 or self.groups < 1 or self.experts % self.groups != 0:
-            raise ValueError(f"{prefix}: {self.experts} experts do not form {self.groups} equal groups")
+        self.identity = int(identity)
+        if self.identity < 0:
+            raise ValueError(f"{prefix}: {self.identity} identity experts")
+        #: What the router chooses among: the experts with matrices, then the identity ones.
+        self.outputs = self.experts + self.identity
+        if self.experts < 1 or self.groups < 1 or self.outputs % self.groups != 0:
+            raise ValueError(f"{prefix}: {self.outputs} router outputs do not form {self.groups} equal groups")
         if not 1 <= self.keep <= self.groups:
             raise ValueError(f"{prefix}: {self.keep} of {self.groups} groups cannot be kept")
-        if not 1 <= self.top <= (self.experts // self.groups) * self.keep:
-            raise ValueError(f"{prefix}: {self.top} experts cannot be taken from {self.keep} groups of {self.experts // self.groups}")
-        if self.experts > 1024 or self.top > 32:
-            raise ValueError(f"{prefix}: the router's kernel takes up to 1,024 experts and 32 per token")
+        if not 1 <= self.top <= (self.outputs // self.groups) * self.keep:
+            raise ValueError(f"{prefix}: {self.top} experts cannot be taken from {self.keep} groups of {self.outputs // self.groups}")
+        if self.outputs > 1024 or self.top > 32:
+            raise ValueError(f"{prefix}: the router's kernel takes up to 1,024 outputs and 32 per token")
+        if router_scores not in ("sigmoid", "softmax"):
+            raise ValueError(f"{prefix}: router scores {router_scores!r} are neither 'sigmoid' nor 'softmax'")
+        self.softmax = router_scores == "softmax"
+        self.correction_name = correction_name or None
+        self.normalise = bool(normalise)
+        self.correction: torch.Tensor | None = None
         self.router_name = router_name
         self.expert_names = tuple(expert_names)
         self.shared = None if shared is None else build_part("feed_forward", shared, self.name(shared_name), runtime)
@@ -82,7 +104,9 @@ class RoutedExperts(FeedForward):
         return self.capturable and (self.shared is None or self.shared.is_capturable())
 
     def tensor_specs(self) -> dict[str, TensorSpec]:
-        specs = {self.name(self.router_name): TensorSpec((self.experts, self.hidden_size))}
+        specs = {self.name(self.router_name): TensorSpec((self.outputs, self.hidden_size))}
+        if self.correction_name:
+            specs[self.name(self.correction_name)] = TensorSpec((self.outputs,), init="zeros")
         for index in range(self.experts):
             specs[self._expert(index, 1)] = TensorSpec((self.expert_size, self.hidden_size))
             specs[self._expert(index, 2)] = TensorSpec((self.expert_size, self.hidden_size))
@@ -102,6 +126,8 @@ class RoutedExperts(FeedForward):
 
     def load(self, tensors: Mapping[str, torch.Tensor]) -> None:
         self.router = tensors[self.name(self.router_name)].contiguous()
+        if self.correction_name:
+            self.correction = tensors[self.name(self.correction_name)].to(torch.float32).contiguous()
         if self.shared_gate_name:
             # The shared expert's gate is one more row of the router's matrix: one product for both.
             self.router = torch.cat([self.router, tensors[self.shared_gate_name].reshape(1, -1)], dim=0).contiguous()
@@ -119,9 +145,12 @@ class RoutedExperts(FeedForward):
     def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
         ops = self.runtime.ops
         taken, weights, gate = ops.moe_route(x, self.router, top=self.top, groups=self.groups, keep=self.keep,
-                                             scale=self.route_scale, experts=self.experts)
+                                             scale=self.route_scale, experts=self.outputs, softmax=self.softmax,
+                                             correction=self.correction, normalise=self.normalise)
         grouping = ops.moe_grouping(taken, self.experts, x.dtype, self.hidden_size, self.expert_size)
         units = ops.moe_expert_units(x, self.gate_up, taken, self.rule, grouping)
         outputs = ops.moe_expert_outputs(units, self.down, taken, grouping)
         extra = self.shared.forward(x, ctx) if self.shared is not None else None
+        if self.identity:
+            return ops.moe_combine(outputs, weights, extra, gate, x.dtype, taken=taken, experts=self.experts, rows=x)
         return ops.moe_combine(outputs, weights, extra, gate, x.dtype)

@@ -19,8 +19,9 @@ class SwiGLU(FeedForward):
 
     ``rule = (steepness, limit, up_shift)`` makes it another gated unit: with ``g = min(gate(x),
     limit)`` and ``u = clamp(up(x), -limit, limit)`` where ``limit > 0``, ``down(g * sigmoid(steepness
-    * g) * (u + up_shift))``; the default ``(1, 0, 0)`` is SwiGLU.  ``names``: the three matrices'
-    tensor names under the part's prefix."""
+    * g) * (u + up_shift))``; the default ``(1, 0, 0)`` is SwiGLU.  A fourth number ``cubic`` makes the
+    gate ``g * sigmoid(steepness * (g + cubic * g^3))``; ``ops.GELU_TANH_RULE`` is the tanh form of GELU
+    on the gate.  ``names``: the three matrices' tensor names under the part's prefix."""
 
     def __init__(self, prefix: str, runtime: Runtime, *, hidden_size: int, intermediate_size: int,
                  rule: tuple[float, float, float] = (1.0, 0.0, 0.0),

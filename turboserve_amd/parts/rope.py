@@ -23,10 +23,19 @@ def rotary_tables(capacity: int, head_dim: int, theta: float, factor: float) -> 
 
 
 def normed_store(runtime: Runtime, qkv, num_heads, num_kv_heads, head_dim, value_dim, ctx, cache: PagedKVView, slots,
-                 head_norm: tuple | None, cos, sin):
+                 head_norm: tuple | None, cos, sin, span_norm: tuple | None = None):
     """The store of a mixer that asked for more than an encoding alone does: a norm per q and k
     head (``head_norm = (q_gain, k_gain, eps, gain_offset)``) and values of a width of their own,
-    with the rotation by ``cos``/``sin`` where given, all in one pass (``ops.head_norm_store``)."""
+    with the rotation by ``cos``/``sin`` where given, all in one pass (``ops.head_norm_store``); or
+    a norm over all q heads at once and all k heads at once (``span_norm``, the same four with
+    gains of the projections' full sizes; ``ops.span_norm_store``, which rotates nothing)."""
+    if span_norm is not None:
+        if head_norm is not None or cos is not None:
+            raise ValueError("a norm over the whole projection goes with no per-head norm and no rotation")
+        q_gain, k_gain, eps, gain_offset = span_norm
+        return runtime.ops.span_norm_store(
+            qkv, cache.k, cache.v, q_gain, k_gain, eps, slots, ctx.num_tokens, num_heads, num_kv_heads, head_dim, value_dim,
+            cache.block_size, runtime.dtype, gain_offset=gain_offset)
     q_gain, k_gain, eps, gain_offset = head_norm if head_norm is not None else (None, None, 0.0, 0.0)
     return runtime.ops.head_norm_store(
         qkv, cache.k, cache.v, q_gain, k_gain, eps, ctx.positions, slots, num_heads, num_kv_heads, head_dim, value_dim,
@@ -91,12 +100,12 @@ class RotaryEncoding(PositionEncoding):
         self.capacity = target
 
     def encode_and_store(self, qkv, num_heads, num_kv_heads, head_dim, ctx, cache: PagedKVView, *,
-                         value_dim: int | None = None, head_norm: tuple | None = None):
+                         value_dim: int | None = None, head_norm: tuple | None = None, span_norm: tuple | None = None):
         self.ensure_capacity(ctx.max_context_len)
         slots = ctx.slot_mapping[cache.group] if cache.writable else None
-        if head_norm is not None or (value_dim is not None and value_dim != head_dim):
+        if head_norm is not None or span_norm is not None or (value_dim is not None and value_dim != head_dim):
             return normed_store(self.runtime, qkv, num_heads, num_kv_heads, head_dim, value_dim or head_dim, ctx, cache,
-                                slots, head_norm, self.cos, self.sin)
+                                slots, head_norm, self.cos, self.sin, span_norm)
         return self.runtime.ops.rope_store(
             qkv, cache.k, cache.v, self.cos, self.sin, ctx.positions, slots,
             num_heads, num_kv_heads, head_dim, cache.block_size, ctx.max_context_len - 1, self.runtime.dtype,
@@ -113,12 +122,32 @@ class NoPositionEncoding(PositionEncoding):
         super().__init__(prefix, runtime)
 
     def encode_and_store(self, qkv, num_heads, num_kv_heads, head_dim, ctx, cache: PagedKVView, *,
-                         value_dim: int | None = None, head_norm: tuple | None = None):
+                         value_dim: int | None = None, head_norm: tuple | None = None, span_norm: tuple | None = None):
         slots = ctx.slot_mapping[cache.group] if cache.writable else None
-        if head_norm is not None or (value_dim is not None and value_dim != head_dim):
+        if head_norm is not None or span_norm is not None or (value_dim is not None and value_dim != head_dim):
             return normed_store(self.runtime, qkv, num_heads, num_kv_heads, head_dim, value_dim or head_dim, ctx, cache,
-                                slots, head_norm, None, None)
+                                slots, head_norm, None, None, span_norm)
         return self.runtime.ops.rope_store(
             qkv, cache.k, cache.v, None, None, ctx.positions, slots,
             num_heads, num_kv_heads, head_dim, cache.block_size, ctx.max_context_len - 1, self.runtime.dtype,
         )
+
+
+@register_position_encoding("distance_slopes")
+class DistanceSlopes(NoPositionEncoding):
+    """Positions enter the scores only: the score of key ``j`` for the query at ``i`` of head ``h`` (of
+    ``H``) loses ``m_h (i - j)``, ``m_h = 2^(-exponent (h + 1) / H)``.  Queries and keys are stored as
+    projected."""
+
+    shareable = True
+
+    def __init__(self, prefix: str, runtime: Runtime, *, exponent: float = 8.0) -> None:
+        super().__init__(prefix, runtime)
+        self.exponent = float(exponent)
+        self._slopes: dict[int, torch.Tensor] = {}
+
+    def score_slopes(self, num_heads: int) -> torch.Tensor:
+        if num_heads not in self._slopes:
+            values = [2.0 ** (-self.exponent * (h + 1) / num_heads) for h in range(num_heads)]
+            self._slopes[num_heads] = torch.tensor(values, dtype=torch.float32, device=self.runtime.device)
+        return self._slopes[num_heads]

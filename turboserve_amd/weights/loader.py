@@ -189,6 +189,13 @@ def iter_checkpoint_tensors(files: list[Path]) -> Iterator[tuple[str, torch.Tens
         yield name, entry.read()
 
 
+def shape_fits(stored: Iterable[int], expected: Iterable[int]) -> bool:
+    """Whether a stored tensor's shape is the one a spec expects; a dimension the spec gives as -1
+    is the checkpoint's to choose (the part checks it against its other tensors when it loads)."""
+    stored, expected = tuple(stored), tuple(expected)
+    return len(stored) == len(expected) and all(want in (-1, have) for have, want in zip(stored, expected))
+
+
 def kept_dtype(stored: torch.dtype, spec: TensorSpec, dtype: torch.dtype) -> torch.dtype | None:
     """The type the run keeps a tensor of ``spec`` in that the checkpoint stores as ``stored``
     (floats in the run's dtype, integer tables as int32, a 32-bit tensor whose spec says so
@@ -262,7 +269,7 @@ def load_tensors(
         if name in found:
             report.unexpected.append(f"{raw_name} (given twice)")
             continue
-        if tuple(entry.shape) != tuple(spec.shape):
+        if not shape_fits(entry.shape, spec.shape):
             report.wrong_shape.append(f"{name}: model has {tuple(spec.shape)}, checkpoint has {tuple(entry.shape)}")
             continue
         kept = kept_dtype(entry.dtype, spec, dtype)

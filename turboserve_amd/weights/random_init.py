@@ -37,6 +37,12 @@ def describe_model(config_data: Mapping[str, Any]):
     return config, DecoderModel(arch.build_plan(config), runtime)
 
 
+def _sized(name: str, spec: TensorSpec) -> None:
+    if any(size < 0 for size in spec.shape):
+        raise ValueError(f"{name}: the configuration leaves a size of {spec.shape} to the checkpoint; "
+                         "random weights need it named")
+
+
 def draw_tensors(
     specs: Mapping[str, TensorSpec], seed: int, *, std: float = 0.02, dtype: torch.dtype = torch.float32
 ) -> Iterator[tuple[str, torch.Tensor]]:
@@ -45,6 +51,7 @@ def draw_tensors(
     for name, spec in specs.items():
         if spec.kind == "int":
             raise ValueError(f"{name}: integer tables have no random initialisation")
+        _sized(name, spec)
         if spec.init == "ones":
             yield name, torch.ones(spec.shape, dtype=dtype)
         elif spec.init == "zeros":
@@ -91,6 +98,7 @@ def random_tensors_on_device(model, seed: int, *, std: float = 0.02) -> None:
 
     def make(name: str) -> torch.Tensor:
         spec = specs[name]
+        _sized(name, spec)
         if spec.init == "ones":
             return torch.ones(spec.shape, dtype=runtime.dtype, device=runtime.device)
         if spec.init == "zeros":
