@@ -87,7 +87,7 @@ class DecodeGraphs:
         total = shape.layout.total
         shape.device_ints = torch.zeros(total, dtype=torch.int32, device=self.device)
         shape.host_ints = [torch.zeros(total, dtype=torch.int32).pin_memory() for _ in range(2)]
-        max_context = max(widths) * self.page_size
+        max_context = max(widths, default=1) * self.page_size  # (a model of stateful layers alone has no pages)
         shape.ctx = StepContext(
             num_tokens=batch,
             num_seqs=batch,

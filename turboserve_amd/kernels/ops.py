@@ -1051,8 +1051,8 @@ class Ops:
         _need(q.is_contiguous() and q.numel() >= tokens * q_stride and q_stride >= heads * head_dim,
               "q does not hold [T, q_stride] rows")
         _need(block_table.dim() == 2 and token_seq.numel() == tokens, "block_table [S, MB], token_seq [T]")
-        _need(attention_geometry_error(heads, kv_heads, head_dim) is None,
-              attention_geometry_error(heads, kv_heads, head_dim) or "")
+        _need(1 <= kv_heads and heads % kv_heads == 0 and heads <= 65535 and 1 <= head_dim <= ATTENTION_MAX_HEAD_DIM,
+              f"{heads} query heads on {kv_heads} KV heads of {head_dim} elements are outside what the kernel takes")
         out = self.rows_buffer(tokens, heads * value_dim, q.dtype, q.device)
         _check(self.core.ts_paged_attention_generic(
             _ptr(out), _ptr(q), q_stride, _ptr(k_pages), _ptr(v_pages), _ptr(block_table),

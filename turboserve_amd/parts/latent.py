@@ -58,9 +58,9 @@ class LatentAttention(Mixer):
         self.wide = self.rank + self.rot_dim
         if min(self.num_heads, self.head_dim, self.rot_dim, self.value_dim, self.rank) < 1 or self.num_heads > 1024:
             raise ValueError(f"{prefix or 'latent attention'}: sizes must be positive and the heads at most 1,024")
-        if self.wide > 512 or self.wide % 2 != 0:
-            raise ValueError(f"{prefix or 'latent attention'}: a cached row of {self.wide} elements is odd or above the "
-                             "512 the attention kernel takes")
+        if self.wide > 512:
+            raise ValueError(f"{prefix or 'latent attention'}: a cached row of {self.wide} elements is above the 512 the "
+                             "attention kernel takes")
         self.rotation = build_part("position_encoding", rotation, prefix, runtime)
         if not 2 <= self.rotation.head_dim <= self.rot_dim:
             raise ValueError(f"{prefix or 'latent attention'}: {self.rotation.head_dim} turned elements do not fit {self.rot_dim}")
@@ -116,6 +116,9 @@ class LatentAttention(Mixer):
             ctx.block_tables[cache.group], ctx.token_seq, ctx.positions, self.num_heads, self.scale, None,
             value_dim=self.rank)
         values = ops.per_head_rows(attended.view(tokens * self.num_heads, self.rank), self.up_v)
-        heads_out = ops.rows_buffer(tokens, self.num_heads * self.value_dim, dtype, x.device)
-        heads_out.copy_(values.view(tokens, self.num_heads * self.value_dim))
+        heads_out = values.view(tokens, self.num_heads * self.value_dim)
+        if dtype != torch.float32:  # the products' 32-bit results, rounded once for the output matrix
+            rounded = ops.rows_buffer(tokens, self.num_heads * self.value_dim, dtype, x.device)
+            rounded.copy_(heads_out)
+            heads_out = rounded
         return ops.linear(heads_out, self.o_weight, for_residual=True)
