@@ -33,7 +33,7 @@ and one 2,048-token prompt), ``--shape 32b --batch 64 --fill-hbm`` (a cache pool
 free memory), ``--closed-loop C [--sampled]`` (the reference's serving profile driven offline: 256
 requests of 128..1,024 tokens in and 64..512 out, C in flight; the library's products run at a
 few step sizes that are all timed at start-up, about 70 s the first time), ``--attention-prefill T[,CTX]`` (the
-prefill attention kernel alone), ``--sample-kernel ROWS`` (the sampling kernel alone), ``--hbm-read`` (a kernel that only reads: what the memory gives), ``--only-prefill [TOKENS]`` (one prompt's prefill alone, 2,048 tokens or TOKENS), ``--designs [2k,4k]`` (the Sisisun design beside a Qwen2 model of equal layer sizes: prefill and decode), ``--kernel-shares TRACE.csv`` (no GPU: the per-kernel table of a
+prefill attention kernel alone), ``--sample-kernel ROWS`` (the sampling kernel alone), ``--hbm-read`` (a kernel that only reads: what the memory gives), ``--only-prefill [TOKENS]`` (one prompt's prefill alone, 2,048 tokens or TOKENS), ``--designs [2k,4k]`` (the Sisisun design beside a Qwen2 model of equal layer sizes: prefill and decode; with ``--design kisadra`` the Kisadra design beside Sisisun), ``--kernel-shares TRACE.csv`` (no GPU: the per-kernel table of a
 ``rocprofv3 --kernel-trace`` of any of these runs).
 """
 
@@ -124,6 +124,8 @@ def parse_args(argv: list[str] | None = None) -> argparse.Namespace:
                    help="prefill and decode of the Sisisun design (random weights) at layer sizes that resemble a real "
                         "model's (2k, 4k: the width), beside a Qwen2 model of the same width, heads, feed-forward and "
                         "number of layer runs; prints one JSON object and exits")
+    p.add_argument("--design", choices=["sisisun", "kisadra"], default="sisisun",
+                   help="which design --designs measures: sisisun beside Qwen2, or kisadra beside sisisun")
     return p.parse_args(argv)
 
 
@@ -498,6 +500,45 @@ def design_pair(size: str) -> tuple[dict, dict]:
     return sisisun, qwen2
 
 
+#: ``--designs --design kisadra``: the Kisadra configuration of a size (its three mixers twice over, dense and routed
+#: feed-forwards in turn, the first two layers run twice) beside the Sisisun configuration of that size.
+def kisadra_pair(size: str) -> tuple[dict, dict]:
+    width, heads, kv, ff, experts, top, expert_ff, rank = {
+        "2k": (2048, 16, 4, 8192, 32, 4, 1024, 256),
+        "4k": (4096, 32, 8, 14336, 64, 6, 1408, 384),
+    }[size]
+    mixers = [
+        ("attention", {"heads": heads, "kv_heads": kv, "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "mask": {"size": 1024}}),
+        ("latent_attention", {"heads": heads, "dim": 128, "rot_dim": 64, "vdim": 128, "kv_rank": rank, "scale": 192 ** -0.5,
+                              "rot": {"base": 10000.0, "dims": 64}}),
+        ("gla", {"heads": heads, "dim": 128, "vdim": 128, "tau": 16.0, "rank": 16}),
+    ]
+    dense = {"kind": "dense", "ff": ff}
+    routed = {"kind": "moe", "expert": {"ff": expert_ff, "limit": 7.0}, "router": {"experts": experts, "identity": 2, "top": top}}
+    layers = [{"type": mixers[i % 3][0], "mixer": mixers[i % 3][1], "mlp": dense if i % 2 == 0 else routed} for i in range(6)]
+    kisadra = {"architecture": "Kisadra", "vocab": 32000, "width": width, "norm": {"eps": 1e-6}, "layers": layers,
+               "loop": {"start": 0, "stop": 2, "times": 2}}
+    return kisadra, design_pair(size)[0]
+
+
+def mixer_work(mixer, batch: int, context: int, prompt: int) -> tuple[float, float]:
+    """``(elements a decode step of `batch` requests at `context` tokens reads from the cache or state,
+    multiply-adds x 2 of a prompt of `prompt` tokens inside the mixer beside its plain projections)``."""
+    kind = type(mixer).__name__
+    if kind == "GatedLinearAttention":
+        state = mixer.num_heads * mixer.head_dim * mixer.value_dim
+        return batch * 2 * state * 2.0, 4.0 * prompt * state  # 32-bit state read and written: 2 x 2 run-dtype elements
+    if kind == "LatentAttention":
+        seen = prompt * (prompt + 1) / 2
+        per_head = 2.0 * prompt * mixer.rank * (mixer.head_dim + mixer.value_dim)
+        return batch * context * mixer.wide, mixer.num_heads * (2.0 * seen * (mixer.wide + mixer.rank) + per_head)
+    chunk = getattr(mixer, "chunk", None) or 10 ** 9
+    seen = sum(i % chunk + 1 for i in range(prompt))
+    visible = (context - 1) % chunk + 1
+    width = mixer.head_dim + mixer.value_dim
+    return batch * visible * mixer.num_kv_heads * width, 2.0 * seen * mixer.num_heads * width
+
+
 def active_weight_elements(model, batch: int, *, per_token: bool = False) -> float:
     """Elements of the weights a step of ``batch`` tokens reads: every tensor of every layer run
     once, but of a routed feed-forward's experts only as many as ``batch`` tokens can take.  With
@@ -519,7 +560,7 @@ def active_weight_elements(model, batch: int, *, per_token: bool = False) -> flo
     return total + head
 
 
-def run_designs(sizes: list[str], dtype_name: str, steps: int, warmup: int) -> dict:
+def run_designs(sizes: list[str], dtype_name: str, steps: int, warmup: int, design: str = "sisisun") -> dict:
     """Prefill (2,048 tokens, best of three) and decode (8 requests at 2,048 tokens of context)
     of both designs at each size, through ``LLMEngine``; with the bytes a decode step reads and
     the multiply-adds a prompt takes, so that both can be set against what the device gives."""
@@ -536,7 +577,8 @@ def run_designs(sizes: list[str], dtype_name: str, steps: int, warmup: int) -> d
     for size in sizes:
         size, _, only = size.partition(":")  # "2k:qwen2": that design alone; "2k:qwen2:prefill": that phase alone (for profiles)
         only, _, phase = only.partition(":")
-        for label, shape in zip(("sisisun", "qwen2"), design_pair(size)):
+        labels, pair = (("kisadra", "sisisun"), kisadra_pair(size)) if design == "kisadra" else (("sisisun", "qwen2"), design_pair(size))
+        for label, shape in zip(labels, pair):
             if only and only != label:
                 continue
             runtime = make_runtime(dtype, "cuda:0")
@@ -545,12 +587,10 @@ def run_designs(sizes: list[str], dtype_name: str, steps: int, warmup: int) -> d
             decode = run_decode(model, config, batch, context - 1, steps=steps, warmup=warmup) if phase != "prefill" \
                 else {"mean_context": context, "step_seconds": float("inf"), "tokens_per_s": 0.0}
             seconds = run_prefill(model, config, prompt, tune=False) if phase != "decode" else float("inf")
-            needs = [need for need in model.cache_needs() if need is not None]
-            kv_elements = sum(n.num_kv_heads * (n.head_dim + n.value_width) for n in needs)
-            read = (active_weight_elements(model, batch) + batch * decode["mean_context"] * kv_elements) * itemsize
-            heads_per_kv = [model.blocks[c.layer].mixer.num_heads // model.blocks[c.layer].mixer.num_kv_heads for c in model.plan.schedule]
+            work = [mixer_work(model.blocks[c.layer].mixer, batch, int(decode["mean_context"]), prompt) for c in model.plan.schedule]
+            read = (active_weight_elements(model, batch) + sum(w[0] for w in work)) * itemsize
             flops = 2.0 * prompt * (active_weight_elements(model, prompt, per_token=True) - model.plan.vocab_size * model.plan.hidden_size) \
-                + sum(4.0 * prompt * prompt / 2 * n.num_kv_heads * g * (n.head_dim + n.value_width) / 2 for n, g in zip(needs, heads_per_kv))
+                + sum(w[1] for w in work)
             out[f"{size}_{label}"] = {
                 "layer_runs": len(model.plan.schedule), "parameters_M": round(model.num_parameters() / 1e6, 1),
                 "prefill_ms": round(seconds * 1e3, 3), "prefill_tokens_per_s": round(prompt / seconds, 1),
@@ -602,7 +642,7 @@ def main(argv: list[str] | None = None) -> int:
         print(json.dumps(run_attention_prefill(SHAPES[args.shape][1], sizes[0], sizes[-1])))
         return 0
     if args.designs:
-        print(json.dumps(run_designs(args.designs.split(","), args.dtype, min(args.steps, 32), min(args.warmup, 8))))
+        print(json.dumps(run_designs(args.designs.split(","), args.dtype, min(args.steps, 32), min(args.warmup, 8), args.design)))
         return 0
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this engine (single-GPU by design)")

@@ -184,6 +184,52 @@ def test_the_state_walk_whole_and_in_pieces(ops, heads, dim, vdim, low, lengths)
         torch.testing.assert_close(state.cpu(), want_state, rtol=2e-4, atol=2e-4)
 
 
+@pytest.mark.parametrize("heads,kv_heads,dim,vdim,in_keys,page,rule", [
+    (4, 2, 16, 8, False, 16, dict(chunk=20, sinks=1.0, slopes=True)),
+    (6, 2, 32, 32, False, 32, dict(chunk=64, sinks=1.0, slopes=True)),
+    (16, 1, 80, 64, True, 16, dict()),
+    (8, 1, 320, 256, True, 16, dict()),
+    (70, 1, 40, 24, True, 8, dict(window=33)),
+    (8, 4, 128, 128, False, 16, dict(chunk=1024, sinks=2.0, slopes=True, softcap=5.0)),
+    (2, 2, 48, 104, False, 64, dict(window=100, sinks=0.5)),
+])
+def test_the_tiled_attention_kernel_against_the_generic_one(ops, heads, kv_heads, dim, vdim, in_keys, page, rule):
+    """bfloat16 on the matrix cores against the one-wavefront-per-row kernel on the same pages: prompt
+    portions that start in the middle of a request, beside single tokens whose keys are shared out over
+    several workgroups; every score rule; values in pages of their own or inside the key rows."""
+    g = torch.Generator().manual_seed(heads * 100 + dim)
+    query_lens = [130, 64, 3, 1, 1, 1]
+    contexts = [400, 64, 1100, 1500, 1, 65]
+    pages_of = [-(-c // page) for c in contexts]
+    total_pages = sum(pages_of) + 3
+    order = torch.randperm(total_pages, generator=g).tolist()
+    table = torch.zeros((len(contexts), max(pages_of)), dtype=torch.int32)
+    for s, n in enumerate(pages_of):
+        table[s, :n] = torch.tensor([order.pop() for _ in range(n)])
+    k_pages = torch.randn(total_pages, kv_heads, page, dim, generator=g).to(torch.bfloat16)
+    v_pages = None if in_keys else torch.randn(total_pages, kv_heads, vdim, page, generator=g).to(torch.bfloat16)
+    tokens = sum(query_lens)
+    q = (0.5 * torch.randn(tokens, heads * dim, generator=g)).to(torch.bfloat16)
+    starts = torch.tensor([0, *torch.tensor(query_lens).cumsum(0).tolist()], dtype=torch.int32)
+    token_seq = torch.repeat_interleave(torch.arange(len(query_lens)), torch.tensor(query_lens)).to(torch.int32)
+    positions = torch.cat([torch.arange(c - n, c) for c, n in zip(contexts, query_lens)]).to(torch.int32)
+    slopes = torch.tensor(plain.distance_slopes(heads), dtype=torch.float32, device=DEV) if rule.get("slopes") else None
+    scale = dim ** -0.5
+    dev = lambda t: None if t is None else t.to(DEV)
+    want = ops.paged_attention_generic(dev(q), heads * dim, dev(k_pages), dev(v_pages), dev(table), dev(token_seq), dev(positions),
+                                       heads, scale, rule.get("window"), slopes, rule.get("softcap", 0.0), chunk=rule.get("chunk"),
+                                       sinks=rule.get("sinks", 0.0), value_dim=vdim if in_keys else None).float().cpu()
+    tiles = torch.tensor(ops.attention_tile_list(query_lens[:3]), dtype=torch.int32, device=DEV)
+    got = ops.attention_tiles(dev(q), heads * dim, dev(k_pages), dev(v_pages), dev(table), dev(starts),
+                              torch.tensor(contexts, dtype=torch.int32, device=DEV), tokens=tokens, heads=heads, scale=scale,
+                              prefill_tiles=tiles, num_prefill_seqs=3, num_decode_seqs=3, max_decode_context=1536,
+                              window=rule.get("window"), chunk=rule.get("chunk"), sinks=rule.get("sinks", 0.0), slopes=slopes,
+                              softcap=rule.get("softcap", 0.0), value_dim=vdim if in_keys else None).float().cpu()
+    assert torch.isfinite(got).all()
+    # Both round probabilities' products differently (bfloat16 probabilities here); outputs are averages of values of size one.
+    torch.testing.assert_close(got, want, rtol=2e-2, atol=2e-2)
+
+
 # ---------------------------------------------------------------------------------------------
 # mechanisms alone: one-layer models
 # ---------------------------------------------------------------------------------------------
@@ -397,7 +443,7 @@ CHUNK = 40
 
 def marked_config(kind: str) -> dict:
     first = {"chunks": kt.layer(kt.attention(2, 1, 32, 32, CHUNK, scale=0.8), None),
-             "latent": kt.layer(kt.latent(2, 32, 4, 32, 32, scale=0.8), None),
+             "latent": kt.layer(kt.latent(2, 32, 8, 32, 32, scale=0.8), None),
              "state": kt.layer(kt.gla(2, 32, 32, 64.0, 4), None)}[kind]
     return {"architecture": "Kisadra", "vocab": 64, "width": 64, "norm": {"eps": 1e-6},
             "layers": [first, kt.layer(kt.gla(1, 8, 8, 2.0, 2), kt.dense(64))], "loop": {"start": 1, "stop": 1, "times": 1}}
@@ -444,9 +490,9 @@ def marked_model(folder, kind: str, dtype: torch.dtype):
         up_v = torch.zeros(2, 32, 32)
         up_v[:, :16, 16:] = 4.0 * torch.randn(16, 16, generator=g)
         tensors["l0.mix.uv"] = up_v.reshape(64, 32)
-        query = torch.zeros(2, 36, 64)
+        query = torch.zeros(2, 40, 64)
         query[:, :16, :32] = 3.0 * down[:16, :32] @ (address[:, None] * asking[None, :] / (asking @ asking))
-        tensors["l0.mix.q"] = query.reshape(72, 64)
+        tensors["l0.mix.q"] = query.reshape(80, 64)
         tensors["l0.mix.dkv.norm"].fill_(1.0)
     else:
         tensors["l0.mix.q"][:, 32:] = 0

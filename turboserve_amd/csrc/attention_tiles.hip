@@ -1,0 +1,426 @@
+// Paged attention on the matrix cores for the score rules and cache shapes the head-size-specialised
+// kernels do not take (bfloat16): keys and values of different widths, values that are the first
+// elements of the key rows themselves (a layer that caches one vector per token), a bias on the
+// scores that is linear in the distance, chunks of positions, a window, sinks in the softmax's
+// denominator.  Same arithmetic as ts_paged_attention_generic: scores, bias, masks and softmax in
+// 32-bit; products of bfloat16 operands accumulated in 32-bit.
+//
+// A workgroup of four wavefronts owns 64 query rows and walks the keys they may see in tiles of 64:
+//   * prompt portions: the rows are 64 consecutive tokens of one request and one query head (the
+//     tile list comes from the host);
+//   * single tokens: the rows are the query heads of one KV head for one request's token; the keys
+//     are shared out over `splits` workgroups whose unnormalised sums ts_attention_tiles_combine
+//     puts together.
+// A tile of keys goes global memory -> registers -> LDS ([key][Dk], and the values as [Dv][key]: from
+// the transposed value pages as they are, or turned while being staged when they lie in the key
+// rows); the next tile's loads are in flight while this one is computed.  Per wavefront: S (16 rows
+// x 64 keys) = Q K^T by v_mfma_f32_16x16x32_bf16, online softmax in the accumulator layout, P
+// through LDS into the operand layout, O += P V.
+//
+// Sizes: Dk (up to 384) and Dv (up to 256) multiples of 8; pages of 8 tokens or more (a multiple of 8).
+#include "common.hpp"
+
+typedef __bf16 fa_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float fa_f32x4 __attribute__((ext_vector_type(4)));
+
+#define FA_ROWS 64
+#define FA_KEYS 64
+#define FA_THREADS 256
+#define FA_PAD 8  // elements of padding behind an LDS row
+
+struct FaRule {
+  float scale;
+  float softcap;
+  float sinks;
+  int window;
+  int chunk;
+};
+
+__device__ __forceinline__ int fa_lowest(int p, int window, int chunk) {
+  int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+  if (chunk > 0) lo = max(lo, (p / chunk) * chunk);
+  return lo;
+}
+
+// KD: 32-element pieces of a key row (Dk rounded up), VD: 16-element pieces of a value row.
+// SINGLE: the single-token layout.  VALUES_IN_KEYS: no value pages.
+template <int KD, int VD, bool SINGLE, bool VALUES_IN_KEYS>
+__global__ void __launch_bounds__(FA_THREADS)
+attention_tiles_kernel(uint16_t* __restrict__ out, float* __restrict__ partial_o, float* __restrict__ partial_ml,
+                       const uint16_t* __restrict__ q, long q_stride, const uint16_t* __restrict__ k_pages,
+                       const uint16_t* __restrict__ v_pages, const int* __restrict__ block_table, int table_width,
+                       const int* __restrict__ query_start_loc, const int* __restrict__ context_lens,
+                       const int* __restrict__ tiles, int first_seq, int heads, int kv_heads, int dk, int dv,
+                       int block_size, const float* __restrict__ slopes, FaRule rule, int splits) {
+  extern __shared__ __attribute__((aligned(16))) uint16_t fa_lds[];
+  constexpr int K_ROW = KD * 32 + FA_PAD;       // elements of a staged key row
+  constexpr int V_ROW = FA_KEYS + FA_PAD;       // elements of a staged value column (64 keys)
+  constexpr int P_ROW = FA_KEYS + FA_PAD;
+  uint16_t* ks = fa_lds;                        // [FA_KEYS][K_ROW]
+  uint16_t* vs = ks + FA_KEYS * K_ROW;          // [VD * 16][V_ROW]
+  uint16_t* ps = vs + VD * 16 * V_ROW;          // [4 wavefronts][16][P_ROW]
+
+  const int tid = threadIdx.x;
+  const int wave = tid / TS_WAVE, lane = tid % TS_WAVE;
+  const int r16 = lane % 16, group = lane / 16;
+  const int group_heads = heads / kv_heads;
+
+  // Which rows: (token row of the step, head, position) of row r; rows beyond the tile are idle.
+  int seq, kvh, tile_first_row = 0, tile_rows, head_first = 0;
+  if (SINGLE) {
+    seq = first_seq + blockIdx.x;
+    const int head_tiles = (group_heads + FA_ROWS - 1) / FA_ROWS;
+    kvh = blockIdx.y / head_tiles;
+    head_first = kvh * group_heads + (blockIdx.y % head_tiles) * FA_ROWS;
+    tile_rows = min(FA_ROWS, kvh * group_heads + group_heads - head_first);
+    tile_first_row = query_start_loc[seq];
+  } else {
+    seq = tiles[2 * blockIdx.x];
+    tile_first_row = tiles[2 * blockIdx.x + 1];
+    tile_rows = min(FA_ROWS, query_start_loc[seq + 1] - tile_first_row);
+    head_first = blockIdx.y;
+    kvh = head_first / group_heads;
+  }
+  const int context = context_lens[seq];
+  const int first_position = context - (query_start_loc[seq + 1] - query_start_loc[seq]);
+  auto row_token = [&](int r) { return SINGLE ? tile_first_row : tile_first_row + r; };
+  auto row_head = [&](int r) { return SINGLE ? head_first + r : head_first; };
+  auto row_position = [&](int r) {
+    return SINGLE ? first_position : first_position + (tile_first_row - query_start_loc[seq]) + r;
+  };
+  const int* table = block_table + (size_t)seq * table_width;
+
+  // The keys this workgroup walks: from the lowest any row sees to the highest, in aligned tiles;
+  // of a shared-out walk its share of the tiles.
+  const int p_first = row_position(0), p_last = row_position(tile_rows - 1);
+  const int key_lo = fa_lowest(p_first, rule.window, rule.chunk);
+  int tile_begin = key_lo / FA_KEYS, tile_end = p_last / FA_KEYS + 1;
+  if (splits > 1) {
+    const int per = (tile_end - tile_begin + splits - 1) / splits;
+    tile_begin = tile_begin + (int)blockIdx.z * per;
+    tile_end = min(tile_end, tile_begin + per);
+  }
+
+  // The wavefront's queries as first operands: row wave * 16 + r16, elements 32 kd + 8 group ..
+  ts_u32x4 qf[KD];
+  {
+    const int r = wave * 16 + r16;
+    const bool live = r < tile_rows;
+    const uint16_t* src = q + (size_t)row_token(live ? r : 0) * q_stride + (size_t)row_head(live ? r : 0) * dk;
+#pragma unroll
+    for (int kd = 0; kd < KD; ++kd) {
+      const int at = 32 * kd + 8 * group;
+      qf[kd] = (live && at < dk) ? *reinterpret_cast<const ts_u32x4*>(src + at) : ts_u32x4{0u, 0u, 0u, 0u};
+    }
+  }
+  // Per accumulator row i of this lane (row wave * 16 + 4 group + i): position, lowest key, slope.
+  int pos[4], low[4];
+  float slope[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = wave * 16 + 4 * group + i;
+    const bool live = r < tile_rows;
+    pos[i] = live ? row_position(r) : -1;  // an idle row sees nothing
+    low[i] = live ? fa_lowest(pos[i], rule.window, rule.chunk) : 0;
+    slope[i] = (slopes && live) ? slopes[row_head(r)] : 0.f;
+  }
+  fa_f32x4 o[VD];
+#pragma unroll
+  for (int vt = 0; vt < VD; ++vt) o[vt] = fa_f32x4{0.f, 0.f, 0.f, 0.f};
+  float m_run[4], l_run[4];
+  // A sink is a key of score 0 that is always there; where the keys are shared out, the combining
+  // kernel counts it, once.
+  const bool own_sinks = rule.sinks > 0.f && splits == 1;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    m_run[i] = own_sinks ? 0.f : -INFINITY;
+    l_run[i] = own_sinks ? rule.sinks : 0.f;
+  }
+
+  // What this thread fetches of a tile: 16-byte pieces (key, 8 elements) of the keys, and of
+  // paged values pieces (value element, 8 keys).
+  const int k_pieces_row = dk / 8;
+  const int k_pieces = FA_KEYS * k_pieces_row;
+  constexpr int K_MINE = (FA_KEYS * KD * 4 + FA_THREADS - 1) / FA_THREADS;
+  constexpr int V_MINE = (VD * 16 * (FA_KEYS / 8) + FA_THREADS - 1) / FA_THREADS;
+  const int v_pieces = dv * (FA_KEYS / 8);
+  ts_u32x4 k_reg[K_MINE];
+  ts_u32x4 v_reg[VALUES_IN_KEYS ? 1 : V_MINE];
+  const int last_key = context - 1;
+  auto fetch = [&](int tile) __attribute__((always_inline)) {
+    const int key0 = tile * FA_KEYS;
+#pragma unroll
+    for (int j = 0; j < K_MINE; ++j) {
+      const int piece = tid + j * FA_THREADS;
+      // Outside key_lo .. last: a live key again (its page may have been given back, or never taken); masked later.
+      const int key = max(min(key0 + piece / k_pieces_row, last_key), key_lo);
+      const int page = table[key / block_size];
+      const uint16_t* src = k_pages + (((size_t)page * kv_heads + kvh) * block_size + key % block_size) * dk +
+                            8 * (piece % k_pieces_row);
+      k_reg[j] = piece < k_pieces ? *reinterpret_cast<const ts_u32x4*>(src) : ts_u32x4{0u, 0u, 0u, 0u};
+    }
+    if (!VALUES_IN_KEYS) {
+#pragma unroll
+      for (int j = 0; j < V_MINE; ++j) {
+        const int piece = tid + j * FA_THREADS;
+        const int d = piece / (FA_KEYS / 8);
+        const int key = max(min(key0 + 8 * (piece % (FA_KEYS / 8)), last_key & ~7), key_lo & ~7);  // eight keys of one page
+        const int page = table[key / block_size];
+        const uint16_t* src = v_pages + (((size_t)page * kv_heads + kvh) * dv + d) * block_size + key % block_size;
+        v_reg[j] = piece < v_pieces ? *reinterpret_cast<const ts_u32x4*>(src) : ts_u32x4{0u, 0u, 0u, 0u};
+      }
+    }
+  };
+  auto stage = [&]() __attribute__((always_inline)) {
+#pragma unroll
+    for (int j = 0; j < K_MINE; ++j) {
+      const int piece = tid + j * FA_THREADS;
+      if (piece < k_pieces) {
+        const int key = piece / k_pieces_row, at = 8 * (piece % k_pieces_row);
+        *reinterpret_cast<ts_u32x4*>(ks + key * K_ROW + at) = k_reg[j];
+        if (VALUES_IN_KEYS && at < dv) {
+          // The row's first Dv elements are the key's value: turned into the value tile's columns.
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            vs[(at + 2 * e) * V_ROW + key] = (uint16_t)(k_reg[j][e] & 0xffffu);
+            vs[(at + 2 * e + 1) * V_ROW + key] = (uint16_t)(k_reg[j][e] >> 16);
+          }
+        }
+      }
+    }
+    if (!VALUES_IN_KEYS) {
+#pragma unroll
+      for (int j = 0; j < V_MINE; ++j) {
+        const int piece = tid + j * FA_THREADS;
+        if (piece < v_pieces)
+          *reinterpret_cast<ts_u32x4*>(vs + (piece / (FA_KEYS / 8)) * V_ROW + 8 * (piece % (FA_KEYS / 8))) = v_reg[j];
+      }
+    }
+  };
+  // Rows of the staged tiles that the sizes leave unused are read as operands all the same: zero once.
+  for (int i = tid; i < FA_KEYS * K_ROW + VD * 16 * V_ROW; i += FA_THREADS) fa_lds[i] = 0;
+  __syncthreads();
+
+  uint16_t* my_p = ps + wave * 16 * P_ROW;
+  if (tile_begin < tile_end) fetch(tile_begin);
+  for (int tile = tile_begin; tile < tile_end; ++tile) {
+    __syncthreads();  // everyone has read the tile before
+    stage();
+    __syncthreads();
+    if (tile + 1 < tile_end) fetch(tile + 1);  // in flight while this tile is computed
+    const int key0 = tile * FA_KEYS;
+    // S = Q K^T: four tiles of 16 keys.
+    fa_f32x4 s[4];
+#pragma unroll
+    for (int ct = 0; ct < 4; ++ct) s[ct] = fa_f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int kd = 0; kd < KD; ++kd) {
+      if (32 * kd < dk) {
+#pragma unroll
+        for (int ct = 0; ct < 4; ++ct) {
+          const ts_u32x4 kf = *reinterpret_cast<const ts_u32x4*>(ks + (16 * ct + r16) * K_ROW + 32 * kd + 8 * group);
+          s[ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(fa_bf16x8, qf[kd]),
+                                                          __builtin_bit_cast(fa_bf16x8, kf), s[ct], 0, 0, 0);
+        }
+      }
+    }
+    // Scores of this lane: row 4 group + i, key key0 + 16 ct + r16.
+    float tile_max[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) tile_max[i] = -INFINITY;
+#pragma unroll
+    for (int ct = 0; ct < 4; ++ct) {
+      const int key = key0 + 16 * ct + r16;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float v = s[ct][i] * rule.scale;
+        if (rule.softcap > 0.f) v = rule.softcap * tanhf(v / rule.softcap);
+        v = fmaf(slope[i], (float)(key - pos[i]), v);
+        v = (key >= low[i] && key <= pos[i]) ? v : -INFINITY;
+        s[ct][i] = v;
+        tile_max[i] = fmaxf(tile_max[i], v);
+      }
+    }
+    float alpha[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      float v = tile_max[i];
+      v = fmaxf(v, __shfl_xor(v, 1, 64));
+      v = fmaxf(v, __shfl_xor(v, 2, 64));
+      v = fmaxf(v, __shfl_xor(v, 4, 64));
+      v = fmaxf(v, __shfl_xor(v, 8, 64));
+      const float m_new = fmaxf(m_run[i], v);
+      // A row that has seen nothing yet keeps a zero sum: exp(-inf - -inf) must not be formed.
+      alpha[i] = m_new == -INFINITY ? 1.f : expf(m_run[i] - m_new);
+      m_run[i] = m_new;
+    }
+    float sum[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ct = 0; ct < 4; ++ct) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float p = s[ct][i] == -INFINITY ? 0.f : expf(s[ct][i] - m_run[i]);
+        // The probability as the second product sees it: rounded; the denominator counts the same value.
+        const bf16_t rounded = from_float<bf16_t>(p);
+        sum[i] += to_float(rounded);
+        my_p[(4 * group + i) * P_ROW + 16 * ct + r16] = rounded.bits;
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      float v = sum[i];
+      v += __shfl_xor(v, 1, 64);
+      v += __shfl_xor(v, 2, 64);
+      v += __shfl_xor(v, 4, 64);
+      v += __shfl_xor(v, 8, 64);
+      l_run[i] = l_run[i] * alpha[i] + v;
+    }
+#pragma unroll
+    for (int vt = 0; vt < VD; ++vt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) o[vt][i] *= alpha[i];
+    __builtin_amdgcn_s_waitcnt(0xc07f);  // the wavefront's own LDS writes of P have landed (lgkmcnt 0)
+    __builtin_amdgcn_wave_barrier();
+    // O += P V over the tile's 64 keys.
+#pragma unroll
+    for (int kk = 0; kk < FA_KEYS / 32; ++kk) {
+      const ts_u32x4 pf = *reinterpret_cast<const ts_u32x4*>(my_p + r16 * P_ROW + 32 * kk + 8 * group);
+#pragma unroll
+      for (int vt = 0; vt < VD; ++vt) {
+        if (16 * vt < dv) {
+          const ts_u32x4 vf = *reinterpret_cast<const ts_u32x4*>(vs + (16 * vt + r16) * V_ROW + 32 * kk + 8 * group);
+          o[vt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(fa_bf16x8, pf),
+                                                          __builtin_bit_cast(fa_bf16x8, vf), o[vt], 0, 0, 0);
+        }
+      }
+    }
+  }
+
+  // o[vt][i]: row 4 group + i, value element 16 vt + r16.
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = wave * 16 + 4 * group + i;
+    if (r >= tile_rows) continue;
+    if (splits == 1) {
+      const float inv = l_run[i] > 0.f ? 1.f / l_run[i] : 0.f;
+      uint16_t* dst = out + ((size_t)row_token(r) * heads + row_head(r)) * dv;
+#pragma unroll
+      for (int vt = 0; vt < VD; ++vt)
+        if (16 * vt + r16 < dv) dst[16 * vt + r16] = from_float<bf16_t>(o[vt][i] * inv).bits;
+    } else {
+      // Unnormalised sums with the maximum they were taken against: [request, head, split].
+      const size_t slot = ((size_t)blockIdx.x * heads + row_head(r)) * splits + blockIdx.z;
+      float* dst = partial_o + slot * dv;
+#pragma unroll
+      for (int vt = 0; vt < VD; ++vt)
+        if (16 * vt + r16 < dv) dst[16 * vt + r16] = o[vt][i];
+      if (r16 == 0) {
+        partial_ml[2 * slot] = m_run[i];
+        partial_ml[2 * slot + 1] = l_run[i];
+      }
+    }
+  }
+}
+
+// out[request's token, head, :] from the shares of its keys: one block per (request, head).
+__global__ void __launch_bounds__(128)
+attention_tiles_combine_kernel(uint16_t* __restrict__ out, const float* __restrict__ partial_o,
+                               const float* __restrict__ partial_ml, const int* __restrict__ query_start_loc,
+                               int first_seq, int heads, int dv, int splits, float sinks) {
+  const int item = blockIdx.x, h = blockIdx.y;
+  const size_t base = ((size_t)item * heads + h) * splits;
+  float m = sinks > 0.f ? 0.f : -INFINITY;
+  for (int sp = 0; sp < splits; ++sp) m = fmaxf(m, partial_ml[2 * (base + sp)]);
+  float l = sinks > 0.f ? sinks * expf(0.f - m) : 0.f;
+  for (int sp = 0; sp < splits; ++sp) {
+    const float ms = partial_ml[2 * (base + sp)];
+    if (ms != -INFINITY) l += partial_ml[2 * (base + sp) + 1] * expf(ms - m);
+  }
+  const float inv = l > 0.f ? 1.f / l : 0.f;
+  const int row = query_start_loc[first_seq + item];
+  for (int d = threadIdx.x; d < dv; d += blockDim.x) {
+    float acc = 0.f;
+    for (int sp = 0; sp < splits; ++sp) {
+      const float ms = partial_ml[2 * (base + sp)];
+      if (ms != -INFINITY) acc = fmaf(partial_o[(base + sp) * dv + d], expf(ms - m), acc);
+    }
+    out[((size_t)row * heads + h) * dv + d] = from_float<bf16_t>(acc * inv).bits;
+  }
+}
+
+template <int KD, int VD>
+static int tiles_launch(bool single, bool values_in_keys, dim3 grid, hipStream_t stream, uint16_t* out, float* partial_o,
+                        float* partial_ml, const uint16_t* q, long q_stride, const uint16_t* k_pages,
+                        const uint16_t* v_pages, const int* block_table, int table_width, const int* query_start_loc,
+                        const int* context_lens, const int* tiles, int first_seq, int heads, int kv_heads, int dk, int dv,
+                        int block_size, const float* slopes, FaRule rule, int splits) {
+  constexpr size_t lds = (size_t)(FA_KEYS * (KD * 32 + FA_PAD) + VD * 16 * (FA_KEYS + FA_PAD) + 4 * 16 * (FA_KEYS + FA_PAD)) * sizeof(uint16_t);
+  static_assert(lds <= 160 * 1024, "the staged tiles must fit in LDS");
+#define FA_GO(SINGLE, INKEYS)                                                                                          \
+  do {                                                                                                                 \
+    static bool raised = false;                                                                                        \
+    if (!raised) {                                                                                                     \
+      if (hipFuncSetAttribute((const void*)attention_tiles_kernel<KD, VD, SINGLE, INKEYS>,                             \
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)                     \
+        return TS_ERR_LAUNCH;                                                                                          \
+      raised = true;                                                                                                   \
+    }                                                                                                                  \
+    hipLaunchKernelGGL((attention_tiles_kernel<KD, VD, SINGLE, INKEYS>), grid, dim3(FA_THREADS), lds, stream, out,     \
+                       partial_o, partial_ml, q, q_stride, k_pages, v_pages, block_table, table_width, query_start_loc, \
+                       context_lens, tiles, first_seq, heads, kv_heads, dk, dv, block_size, slopes, rule, splits);     \
+  } while (0)
+  if (single && values_in_keys) FA_GO(true, true);
+  else if (single) FA_GO(true, false);
+  else if (values_in_keys) FA_GO(false, true);
+  else FA_GO(false, false);
+#undef FA_GO
+  return ts_launch_status();
+}
+
+// mode 0: prompt portions, `items` tiles (pairs: request, first row) and grid.y = heads;
+// mode 1: `items` requests of one token each from `first_seq` on, their keys shared out over `splits`.
+// out [T, heads, Dv] bfloat16.  v_pages null: the values are the keys' first Dv elements.
+extern "C" int ts_attention_tiles(void* out, void* partial_o, void* partial_ml, const void* q, long q_stride,
+                                  const void* k_pages, const void* v_pages, const int* block_table, int table_width,
+                                  const int* query_start_loc, const int* context_lens, const int* tiles, int items,
+                                  int first_seq, int heads, int kv_heads, int dk, int dv, int block_size, float scale,
+                                  float softcap, int window, int chunk, float sinks, const float* slopes, int mode,
+                                  int splits, hipStream_t stream) {
+  if (items == 0) return TS_OK;
+  if (!out || !q || !k_pages || !block_table || !query_start_loc || !context_lens) return TS_ERR_ARG;
+  if (mode == 0 && (!tiles || splits != 1)) return TS_ERR_ARG;
+  if (mode == 1 && splits > 1 && (!partial_o || !partial_ml)) return TS_ERR_ARG;
+  if (mode < 0 || mode > 1 || splits < 1 || splits > 65535) return TS_ERR_ARG;
+  if (heads < 1 || kv_heads < 1 || heads % kv_heads != 0 || heads > 65535) return TS_ERR_SHAPE;
+  if (dk < 8 || dk > 384 || dk % 8 != 0 || dv < 8 || dv > 256 || dv % 8 != 0 || block_size < 8 || block_size % 8 != 0)
+    return TS_ERR_SHAPE;
+  if (!v_pages && dv > dk) return TS_ERR_SHAPE;
+  if ((((uintptr_t)q | (uintptr_t)k_pages | (uintptr_t)v_pages) & 15) != 0 || (q_stride % 8) != 0) return TS_ERR_ARG;
+  const FaRule rule = {scale, softcap, sinks, window, chunk};
+  const int group_heads = heads / kv_heads;
+  const dim3 grid(items, mode == 0 ? heads : kv_heads * ((group_heads + FA_ROWS - 1) / FA_ROWS), splits);
+  const bool single = mode == 1, in_keys = v_pages == nullptr;
+  const int kd = (dk + 31) / 32, vd = (dv + 15) / 16;
+#define FA_SIZE(KD, VD)                                                                                                 \
+  return tiles_launch<KD, VD>(single, in_keys, grid, stream, (uint16_t*)out, (float*)partial_o, (float*)partial_ml,     \
+                              (const uint16_t*)q, q_stride, (const uint16_t*)k_pages, (const uint16_t*)v_pages,         \
+                              block_table, table_width, query_start_loc, context_lens, tiles, first_seq, heads, kv_heads, \
+                              dk, dv, block_size, slopes, rule, splits)
+  if (kd <= 2 && vd <= 4) FA_SIZE(2, 4);
+  if (kd <= 4 && vd <= 8) FA_SIZE(4, 8);
+  if (kd <= 8 && vd <= 16) FA_SIZE(8, 16);
+  if (kd <= 12 && vd <= 16) FA_SIZE(12, 16);
+#undef FA_SIZE
+  return TS_ERR_SHAPE;
+}
+
+extern "C" int ts_attention_tiles_combine(void* out, const void* partial_o, const void* partial_ml,
+                                          const int* query_start_loc, int items, int first_seq, int heads, int dv,
+                                          int splits, float sinks, hipStream_t stream) {
+  if (items == 0) return TS_OK;
+  if (!out || !partial_o || !partial_ml || !query_start_loc || splits < 1 || heads < 1 || heads > 65535 || dv < 1)
+    return TS_ERR_ARG;
+  hipLaunchKernelGGL(attention_tiles_combine_kernel, dim3(items, heads), dim3(128), 0, stream, (uint16_t*)out,
+                     (const float*)partial_o, (const float*)partial_ml, query_start_loc, first_seq, heads, dv, splits, sinks);
+  return ts_launch_status();
+}

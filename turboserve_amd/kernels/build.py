@@ -38,6 +38,7 @@ MODULES: dict[str, tuple[str, ...]] = {
         "linear_state.hip",
         "moe.hip",
         "attention_generic.hip",
+        "attention_tiles.hip",
         "gemm_plain.hip",
         "gemm_skinny.hip",
         "gemm_tiled.hip",

@@ -70,6 +70,11 @@ _SIGNATURES: dict[str, dict[str, list]] = {
         "ts_paged_attention_generic": [c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int,
                                        c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
                                        c_float, c_float, c_int, c_void_p, c_int, c_float, c_int, c_void_p],
+        "ts_attention_tiles": [c_void_p, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
+                               c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_float, c_int,
+                               c_int, c_float, c_void_p, c_int, c_int, c_void_p],
+        "ts_attention_tiles_combine": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float,
+                                       c_void_p],
         "ts_head_norm_store": [c_void_p, c_long, c_void_p, c_int, c_int, c_long, c_void_p, c_void_p, c_void_p, c_void_p,
                                c_float, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
                                c_int, c_int, c_int, c_void_p],
@@ -1060,6 +1065,82 @@ class Ops:
             block_size, float(scale), float(softcap), int(window or 0), _ptr(slopes) if slopes is not None else None,
             int(chunk or 0), float(sinks), dtype_code(q.dtype), self.stream()),
             "ts_paged_attention_generic")
+        return out
+
+    @staticmethod
+    def tiled_attention_supported(dtype: torch.dtype, head_dim: int, value_dim: int, block_size: int, q_stride: int) -> bool:
+        """Whether :meth:`attention_tiles` takes this geometry: bfloat16, key rows of up to 384 and
+        values of up to 256 elements, both multiples of 8 (16-byte accesses), pages of a multiple of 8
+        tokens, query rows 16 bytes apart or a multiple of that."""
+        return (dtype == torch.bfloat16 and head_dim % 8 == 0 and 8 <= head_dim <= 384 and value_dim % 8 == 0
+                and 8 <= value_dim <= 256 and block_size % 8 == 0 and q_stride % 8 == 0)
+
+    @staticmethod
+    def attention_tile_list(query_lens, rows: int = 64) -> list[list[int]]:
+        """``[request, first row]`` of every tile of ``rows`` consecutive tokens of the requests
+        ``0 .. len(query_lens) - 1`` at the front of a step."""
+        tiles, row = [], 0
+        for request, count in enumerate(query_lens):
+            tiles.extend([request, row + first] for first in range(0, count, rows))
+            row += count
+        return tiles
+
+    def attention_tiles(self, q: torch.Tensor, q_stride: int, k_pages: torch.Tensor, v_pages: torch.Tensor | None,
+                        block_table: torch.Tensor, query_start_loc: torch.Tensor, context_lens: torch.Tensor, *,
+                        tokens: int, heads: int, scale: float, prefill_tiles: torch.Tensor | None, num_prefill_seqs: int,
+                        num_decode_seqs: int, max_decode_context: int, window: int | None = None, chunk: int | None = None,
+                        sinks: float = 0.0, slopes: torch.Tensor | None = None, softcap: float = 0.0,
+                        value_dim: int | None = None) -> torch.Tensor:
+        """What :meth:`paged_attention_generic` computes, for bfloat16, on the matrix cores: the
+        requests that bring several tokens (the first ``num_prefill_seqs``) in tiles of 64 tokens by
+        one head (``prefill_tiles``: int32 ``[n, 2]`` from :meth:`attention_tile_list`), the
+        ``num_decode_seqs`` single tokens behind them with the heads of a KV head as one tile and
+        their keys (at most ``max_decode_context``, a bound the step's shape gives) shared out over
+        several workgroups.  Returns ``[T, heads * Dv]``."""
+        _gpu(q, k_pages, v_pages, block_table, query_start_loc, context_lens, prefill_tiles, slopes)
+        _i32(block_table, "block_table")
+        _i32(query_start_loc, "query_start_loc")
+        _i32(context_lens, "context_lens")
+        _i32(prefill_tiles, "prefill_tiles")
+        _need(q.dtype == torch.bfloat16 and k_pages.dtype == torch.bfloat16 and k_pages.dim() == 4 and k_pages.is_contiguous(),
+              "queries and key pages [NB, Hkv, BS, D] must be bfloat16")
+        _, kv_heads, block_size, head_dim = k_pages.shape
+        if v_pages is not None:
+            _check_pages(k_pages, v_pages, q.dtype, any_value_width=True)
+            value_dim = v_pages.shape[2]
+        _need(value_dim is not None and (v_pages is not None or value_dim <= head_dim), "values inside the keys are their first value_dim elements")
+        _need(self.tiled_attention_supported(q.dtype, head_dim, value_dim, block_size, q_stride), "a geometry the tiled attention kernel does not take")
+        _need(heads % kv_heads == 0 and q.is_contiguous() and q.numel() >= tokens * q_stride and q_stride >= heads * head_dim,
+              "q does not hold [T, q_stride] rows of the heads")
+        _need(block_table.dim() == 2 and query_start_loc.numel() >= num_prefill_seqs + num_decode_seqs + 1, "block_table [S, MB], row ranges [S + 1]")
+        if slopes is not None:
+            _need(slopes.dtype == torch.float32 and slopes.is_contiguous() and slopes.numel() == heads, "slopes must be float32 [heads]")
+        out = self.rows_buffer(tokens, heads * value_dim, q.dtype, q.device)
+        common = (_ptr(q), q_stride, _ptr(k_pages), _ptr(v_pages), _ptr(block_table), block_table.shape[1],
+                  _ptr(query_start_loc), _ptr(context_lens))
+        rule = (float(scale), float(softcap), int(window or 0), int(chunk or 0), float(sinks), _ptr(slopes))
+        if num_prefill_seqs > 0:
+            _need(prefill_tiles is not None and prefill_tiles.dim() == 2 and prefill_tiles.shape[1] == 2, "prefill_tiles [n, 2]")
+            _check(self.core.ts_attention_tiles(_ptr(out), None, None, *common, _ptr(prefill_tiles), prefill_tiles.shape[0], 0,
+                                                heads, kv_heads, head_dim, value_dim, block_size, *rule, 0, 1, self.stream()),
+                   "ts_attention_tiles")
+        if num_decode_seqs > 0:
+            # Workgroups per (request, KV head): enough to give every compute unit one, no more than the
+            # keys have tiles of 64 (a chunk or window bounds what a token sees).
+            seen = max(1, min(max_decode_context, chunk or max_decode_context, window or max_decode_context))
+            head_tiles = kv_heads * (-(-(heads // kv_heads) // 64))
+            splits = max(1, min(-(-seen // 64), -(-self.compute_units // (num_decode_seqs * head_tiles)), 64))
+            partial_o = partial_ml = None
+            if splits > 1:
+                partial_o = torch.empty((num_decode_seqs, heads, splits, value_dim), dtype=torch.float32, device=q.device)
+                partial_ml = torch.empty((num_decode_seqs, heads, splits, 2), dtype=torch.float32, device=q.device)
+            _check(self.core.ts_attention_tiles(_ptr(out), _ptr(partial_o), _ptr(partial_ml), *common, None, num_decode_seqs,
+                                                num_prefill_seqs, heads, kv_heads, head_dim, value_dim, block_size, *rule, 1,
+                                                splits, self.stream()), "ts_attention_tiles")
+            if splits > 1:
+                _check(self.core.ts_attention_tiles_combine(_ptr(out), _ptr(partial_o), _ptr(partial_ml), _ptr(query_start_loc),
+                                                            num_decode_seqs, num_prefill_seqs, heads, value_dim, splits,
+                                                            float(sinks), self.stream()), "ts_attention_tiles_combine")
         return out
 
     @staticmethod

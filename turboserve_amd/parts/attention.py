@@ -12,6 +12,19 @@ from turboserve_amd.parts.base import CacheNeed, Mixer, PagedKV, PagedKVView, Pa
 from turboserve_amd.parts.registry import build_part, register_mixer
 
 
+def tiled_attention(ops, q, q_stride, k_pages, v_pages, table, ctx, **rule) -> torch.Tensor:
+    """A step's attention by ``ops.attention_tiles``: the tile list of the requests that bring several
+    tokens is made once per step and shared by the layers (a recorded step has none: single tokens)."""
+    tiles = None
+    if ctx.num_prefill_seqs > 0:
+        tiles = ctx.derive("attention_tiles_64", lambda step: torch.tensor(
+            ops.attention_tile_list(step.query_lens[:step.num_prefill_seqs]), dtype=torch.int32, device=q.device))
+    return ops.attention_tiles(
+        q, q_stride, k_pages, v_pages, table, ctx.query_start_loc, ctx.context_lens, tokens=ctx.num_tokens,
+        prefill_tiles=tiles, num_prefill_seqs=ctx.num_prefill_seqs, num_decode_seqs=ctx.num_decode_seqs,
+        max_decode_context=min(ctx.max_decode_context_len, table.shape[1] * k_pages.shape[2]), **rule)
+
+
 @register_mixer("gqa_attention")
 class GroupedQueryAttention(Mixer):
     """q/k/v projections (optionally biased), position encoding, cache write, attention of every
@@ -186,8 +199,9 @@ class GroupedQueryAttention(Mixer):
 
         bfloat16 runs use the matrix-core kernels where the geometry allows: one launch for the
         multi-token requests at the front of the batch, one for the single-token requests
-        behind them; every 32-bit run, any other geometry and any position encoding that biases
-        the scores goes through the generic kernel."""
+        behind them; a position encoding that biases the scores, a chunk mask, sinks or values of
+        another width than the keys go through the tiled matrix-core kernel that takes them; every
+        32-bit run and any other geometry goes through the generic kernel."""
         ops = self.runtime.ops
         table = ctx.block_tables[cache.group]
         slopes = self.position.score_slopes(self.num_heads)
@@ -215,6 +229,9 @@ class GroupedQueryAttention(Mixer):
                     ctx.max_decode_context_dev, softcap=self.softcap,
                 )
             return out
+        if ops.tiled_attention_supported(qkv.dtype, self.head_dim, self.value_dim, cache.block_size, q_stride):
+            return tiled_attention(ops, qkv, q_stride, cache.k, cache.v, table, ctx, heads=self.num_heads, scale=self.scale,
+                                   window=self.window, chunk=self.chunk, sinks=self.sinks, slopes=slopes, softcap=self.softcap)
         return ops.paged_attention_generic(
             qkv, q_stride, cache.k, cache.v, table, ctx.token_seq, ctx.positions,
             self.num_heads, self.scale, self.window, slopes, self.softcap, chunk=self.chunk, sinks=self.sinks,

@@ -7,6 +7,7 @@ from collections.abc import Mapping
 
 import torch
 
+from turboserve_amd.parts.attention import tiled_attention
 from turboserve_amd.parts.base import CacheNeed, Mixer, PagedKV, PagedKVView, PartSpec, Runtime, TensorSpec
 from turboserve_amd.parts.registry import build_part, register_mixer
 
@@ -111,10 +112,14 @@ class LatentAttention(Mixer):
         # The plain query parts through the keys' up-projection: what they are against the latent itself.
         carried = ops.per_head_rows(q_plain, self.up_k)
         q_wide[:, :, : self.rank].copy_(carried.view(tokens, self.num_heads, self.rank))
-        attended = ops.paged_attention_generic(
-            q_wide.view(tokens, self.num_heads * self.wide), self.num_heads * self.wide, cache.k, None,
-            ctx.block_tables[cache.group], ctx.token_seq, ctx.positions, self.num_heads, self.scale, None,
-            value_dim=self.rank)
+        stride = self.num_heads * self.wide
+        if ops.tiled_attention_supported(dtype, self.wide, self.rank, cache.block_size, stride):
+            attended = tiled_attention(ops, q_wide.view(tokens, stride), stride, cache.k, None, ctx.block_tables[cache.group],
+                                       ctx, heads=self.num_heads, scale=self.scale, value_dim=self.rank)
+        else:
+            attended = ops.paged_attention_generic(
+                q_wide.view(tokens, stride), stride, cache.k, None, ctx.block_tables[cache.group], ctx.token_seq,
+                ctx.positions, self.num_heads, self.scale, None, value_dim=self.rank)
         values = ops.per_head_rows(attended.view(tokens * self.num_heads, self.rank), self.up_v)
         heads_out = values.view(tokens, self.num_heads * self.value_dim)
         if dtype != torch.float32:  # the products' 32-bit results, rounded once for the output matrix
