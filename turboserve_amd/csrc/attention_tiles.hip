@@ -36,6 +36,24 @@ struct FaRule {
   int chunk;
 };
 
+// Sum and maximum over the 16 lanes that hold one row of an accumulator tile (a row of lanes for
+// the data-parallel moves): every lane returns its row's result.
+__device__ __forceinline__ float row16_sum(float v) {
+  v += lanes_moved<0xB1, 0xF>(0.f, v);   // quad_perm [1,0,3,2]
+  v += lanes_moved<0x4E, 0xF>(0.f, v);   // quad_perm [2,3,0,1]
+  v += lanes_moved<0x141, 0xF>(0.f, v);  // row_half_mirror
+  v += lanes_moved<0x140, 0xF>(0.f, v);  // row_mirror
+  return v;
+}
+
+__device__ __forceinline__ float row16_max(float v) {
+  v = fmaxf(v, lanes_moved<0xB1, 0xF>(v, v));
+  v = fmaxf(v, lanes_moved<0x4E, 0xF>(v, v));
+  v = fmaxf(v, lanes_moved<0x141, 0xF>(v, v));
+  v = fmaxf(v, lanes_moved<0x140, 0xF>(v, v));
+  return v;
+}
+
 __device__ __forceinline__ int fa_lowest(int p, int window, int chunk) {
   int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
   if (chunk > 0) lo = max(lo, (p / chunk) * chunk);
@@ -45,7 +63,7 @@ __device__ __forceinline__ int fa_lowest(int p, int window, int chunk) {
 // KD: 32-element pieces of a key row (Dk rounded up), VD: 16-element pieces of a value row.
 // SINGLE: the single-token layout.  VALUES_IN_KEYS: no value pages.
 template <int KD, int VD, bool SINGLE, bool VALUES_IN_KEYS>
-__global__ void __launch_bounds__(FA_THREADS)
+__global__ void __launch_bounds__(FA_THREADS, (KD <= 4 ? 2 : 1))  // small tiles: two workgroups a compute unit
 attention_tiles_kernel(uint16_t* __restrict__ out, float* __restrict__ partial_o, float* __restrict__ partial_ml,
                        const uint16_t* __restrict__ q, long q_stride, const uint16_t* __restrict__ k_pages,
                        const uint16_t* __restrict__ v_pages, const int* __restrict__ block_table, int table_width,
@@ -137,13 +155,26 @@ attention_tiles_kernel(uint16_t* __restrict__ out, float* __restrict__ partial_o
     l_run[i] = own_sinks ? rule.sinks : 0.f;
   }
 
-  // What this thread fetches of a tile: 16-byte pieces (key, 8 elements) of the keys, and of
-  // paged values pieces (value element, 8 keys).
+  // What this thread fetches of a tile: 16-byte pieces (key, 8 elements) of the keys, and of paged
+  // values pieces (value element, 8 keys); which pieces is the same for every tile.  Key rows whose
+  // first elements are also the values are turned into the value tile's columns while they are
+  // staged, two bytes at a time: there a wavefront's lanes take the 64 keys of one 8-element piece,
+  // so that its LDS writes fall into different banks; otherwise consecutive lanes take consecutive
+  // pieces of a row (whole cache lines).
   const int k_pieces_row = dk / 8;
   const int k_pieces = FA_KEYS * k_pieces_row;
   constexpr int K_MINE = (FA_KEYS * KD * 4 + FA_THREADS - 1) / FA_THREADS;
   constexpr int V_MINE = (VD * 16 * (FA_KEYS / 8) + FA_THREADS - 1) / FA_THREADS;
   const int v_pieces = dv * (FA_KEYS / 8);
+  const int block_mask = block_size - 1, block_shift = __builtin_ctz(block_size);  // pages hold a power of two
+  int k_key[K_MINE], k_at[K_MINE];
+#pragma unroll
+  for (int j = 0; j < K_MINE; ++j) {
+    const int piece = tid + j * FA_THREADS;
+    k_key[j] = VALUES_IN_KEYS ? piece % FA_KEYS : piece / k_pieces_row;
+    k_at[j] = 8 * (VALUES_IN_KEYS ? piece / FA_KEYS : piece % k_pieces_row);
+    if (piece >= k_pieces) k_key[j] = -1;
+  }
   ts_u32x4 k_reg[K_MINE];
   ts_u32x4 v_reg[VALUES_IN_KEYS ? 1 : V_MINE];
   const int last_key = context - 1;
@@ -151,13 +182,11 @@ attention_tiles_kernel(uint16_t* __restrict__ out, float* __restrict__ partial_o
     const int key0 = tile * FA_KEYS;
 #pragma unroll
     for (int j = 0; j < K_MINE; ++j) {
-      const int piece = tid + j * FA_THREADS;
       // Outside key_lo .. last: a live key again (its page may have been given back, or never taken); masked later.
-      const int key = max(min(key0 + piece / k_pieces_row, last_key), key_lo);
-      const int page = table[key / block_size];
-      const uint16_t* src = k_pages + (((size_t)page * kv_heads + kvh) * block_size + key % block_size) * dk +
-                            8 * (piece % k_pieces_row);
-      k_reg[j] = piece < k_pieces ? *reinterpret_cast<const ts_u32x4*>(src) : ts_u32x4{0u, 0u, 0u, 0u};
+      const int key = max(min(key0 + max(k_key[j], 0), last_key), key_lo);
+      const int page = table[key >> block_shift];
+      const uint16_t* src = k_pages + ((((size_t)page * kv_heads + kvh) << block_shift) + (key & block_mask)) * dk + k_at[j];
+      k_reg[j] = k_key[j] >= 0 ? *reinterpret_cast<const ts_u32x4*>(src) : ts_u32x4{0u, 0u, 0u, 0u};
     }
     if (!VALUES_IN_KEYS) {
 #pragma unroll
@@ -165,8 +194,8 @@ attention_tiles_kernel(uint16_t* __restrict__ out, float* __restrict__ partial_o
         const int piece = tid + j * FA_THREADS;
         const int d = piece / (FA_KEYS / 8);
         const int key = max(min(key0 + 8 * (piece % (FA_KEYS / 8)), last_key & ~7), key_lo & ~7);  // eight keys of one page
-        const int page = table[key / block_size];
-        const uint16_t* src = v_pages + (((size_t)page * kv_heads + kvh) * dv + d) * block_size + key % block_size;
+        const int page = table[key >> block_shift];
+        const uint16_t* src = v_pages + ((((size_t)page * kv_heads + kvh) * dv + d) << block_shift) + (key & block_mask);
         v_reg[j] = piece < v_pieces ? *reinterpret_cast<const ts_u32x4*>(src) : ts_u32x4{0u, 0u, 0u, 0u};
       }
     }
@@ -174,9 +203,8 @@ attention_tiles_kernel(uint16_t* __restrict__ out, float* __restrict__ partial_o
   auto stage = [&]() __attribute__((always_inline)) {
 #pragma unroll
     for (int j = 0; j < K_MINE; ++j) {
-      const int piece = tid + j * FA_THREADS;
-      if (piece < k_pieces) {
-        const int key = piece / k_pieces_row, at = 8 * (piece % k_pieces_row);
+      if (k_key[j] >= 0) {
+        const int key = k_key[j], at = k_at[j];
         *reinterpret_cast<ts_u32x4*>(ks + key * K_ROW + at) = k_reg[j];
         if (VALUES_IN_KEYS && at < dv) {
           // The row's first Dv elements are the key's value: turned into the value tile's columns.
@@ -197,8 +225,10 @@ attention_tiles_kernel(uint16_t* __restrict__ out, float* __restrict__ partial_o
       }
     }
   };
-  // Rows of the staged tiles that the sizes leave unused are read as operands all the same: zero once.
-  for (int i = tid; i < FA_KEYS * K_ROW + VD * 16 * V_ROW; i += FA_THREADS) fa_lds[i] = 0;
+  // What the sizes leave unused of the staged tiles is read as operands all the same: zero, once
+  // (the key rows' elements from Dk on, the value rows from Dv on).
+  for (int i = tid; i < FA_KEYS * (K_ROW - dk); i += FA_THREADS) ks[(i / (K_ROW - dk)) * K_ROW + dk + i % (K_ROW - dk)] = 0;
+  for (int i = tid + dv * V_ROW; i < VD * 16 * V_ROW; i += FA_THREADS) vs[i] = 0;
   __syncthreads();
 
   uint16_t* my_p = ps + wave * 16 * P_ROW;
@@ -244,11 +274,7 @@ attention_tiles_kernel(uint16_t* __restrict__ out, float* __restrict__ partial_o
     float alpha[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      float v = tile_max[i];
-      v = fmaxf(v, __shfl_xor(v, 1, 64));
-      v = fmaxf(v, __shfl_xor(v, 2, 64));
-      v = fmaxf(v, __shfl_xor(v, 4, 64));
-      v = fmaxf(v, __shfl_xor(v, 8, 64));
+      const float v = row16_max(tile_max[i]);
       const float m_new = fmaxf(m_run[i], v);
       // A row that has seen nothing yet keeps a zero sum: exp(-inf - -inf) must not be formed.
       alpha[i] = m_new == -INFINITY ? 1.f : expf(m_run[i] - m_new);
@@ -268,12 +294,7 @@ attention_tiles_kernel(uint16_t* __restrict__ out, float* __restrict__ partial_o
     }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      float v = sum[i];
-      v += __shfl_xor(v, 1, 64);
-      v += __shfl_xor(v, 2, 64);
-      v += __shfl_xor(v, 4, 64);
-      v += __shfl_xor(v, 8, 64);
-      l_run[i] = l_run[i] * alpha[i] + v;
+      l_run[i] = l_run[i] * alpha[i] + row16_sum(sum[i]);
     }
 #pragma unroll
     for (int vt = 0; vt < VD; ++vt)

@@ -11,8 +11,8 @@
 // Row of the projection (type T, or `splits` 32-bit partial sums): [H D q | H D k | H Dv v | H Dv gate | R y].
 //
 // ts_linear_state_scan walks the tokens of one piece of a request with the state in registers: a
-// block of 256 threads owns one head and 64 value columns, thread (column c, quarter p) holds rows
-// p, p + 4, p + 8, .. of S[:, c].  Eight tokens at a time are staged in LDS (q, k and the decays,
+// block of 256 threads owns one head and 64 value columns, thread (column c, quarter p) holds a quarter of
+// the rows of S[:, c], one after the other (four rows' staged values are one LDS read).  Eight tokens at a time are staged in LDS (q, k and the decays,
 // which the block computes from y), then every thread updates its rows and leaves its share of o;
 // the four shares of a column meet in LDS.  Three uses:
 //   whole  the piece is all the tokens a request brings; S comes from the request's slot and
@@ -33,12 +33,24 @@
 #define LS_QUARTERS 4   // threads per column
 #define LS_BATCH 8      // tokens staged at a time
 #define LS_MAX_DIM 256  // key channels (one thread each computes a channel's decay)
-#define LS_MAX_LOW 64   // width of y
+#define LS_MAX_LOW 128  // width of y
 
+typedef float ls_f32x4 __attribute__((ext_vector_type(4)));
+
+// The sum of a projection's partial sums, added in split order, eight loads in flight at a time (a
+// loop of load, wait, add would cost a trip to memory per split).
 template <typename P>
 __device__ __forceinline__ float ls_folded(const P* p, int splits, size_t stride) {
-  float s = to_float(p[0]);
-  for (int i = 1; i < splits; ++i) s += to_float(p[(size_t)i * stride]);
+  if (splits == 1) return to_float(p[0]);
+  float s = 0.f;
+  for (int first = 0; first < splits; first += 8) {
+    float v[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = to_float(p[(size_t)min(first + j, splits - 1) * stride]);
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      if (first + j < splits) s += v[j];
+  }
   return s;
 }
 
@@ -58,9 +70,9 @@ linear_state_scan_kernel(float* __restrict__ out, const P* __restrict__ proj, in
                          const int* __restrict__ query_start_loc, int first_seq, const LsPiece* __restrict__ pieces,
                          float* __restrict__ piece_state, float* __restrict__ piece_decay, int heads, int dim, int vdim,
                          int low) {
-  __shared__ float qs[LS_BATCH][LS_MAX_DIM];
-  __shared__ float ks[LS_BATCH][LS_MAX_DIM];
-  __shared__ float as[LS_BATCH][LS_MAX_DIM];
+  __shared__ __attribute__((aligned(16))) float qs[LS_BATCH][LS_MAX_DIM];
+  __shared__ __attribute__((aligned(16))) float ks[LS_BATCH][LS_MAX_DIM];
+  __shared__ __attribute__((aligned(16))) float as[LS_BATCH][LS_MAX_DIM];
   __shared__ float ys[LS_BATCH][LS_MAX_LOW];
   __shared__ float shares[LS_BATCH][LS_QUARTERS][LS_COLS];
   const int item = blockIdx.x, h = blockIdx.y;
@@ -84,18 +96,25 @@ linear_state_scan_kernel(float* __restrict__ out, const P* __restrict__ proj, in
   const float q_scale = rsqrtf((float)dim);
   const size_t per_head = (size_t)dim * vdim;
 
-  // The thread's rows of the state: d = p + 4 r.
+  // The thread's rows of the state: d = p * ROWS + r.
   float s[ROWS];
   const float* from = nullptr;
   if (MODE == 0) from = state + ((size_t)state_slots[seq] * heads + h) * per_head;
   if (MODE == 2) from = piece_state + ((size_t)item * heads + h) * per_head;
 #pragma unroll
   for (int r = 0; r < ROWS; ++r) {
-    const int d = p + LS_QUARTERS * r;
+    const int d = p * ROWS + r;
     s[r] = (from && has_col && d < dim) ? from[(size_t)d * vdim + col] : 0.f;
   }
   // Thread d < dim computes channel d's decay; in local mode it also keeps the product of them.
   float decay_product = 1.f;
+  // Channels from dim up to the four quarters' ROWS are read with the others, four at a time: zero keys
+  // and queries there, once, so that their rows of the state stay zero and add nothing.
+  for (int i = tid; i < LS_BATCH * LS_MAX_DIM; i += blockDim.x) {
+    (&qs[0][0])[i] = 0.f;
+    (&ks[0][0])[i] = 0.f;
+    (&as[0][0])[i] = 0.f;
+  }
 
   for (int base = 0; base < count; base += LS_BATCH) {
     const int n = min(LS_BATCH, count - base);
@@ -133,11 +152,17 @@ linear_state_scan_kernel(float* __restrict__ out, const P* __restrict__ proj, in
       if (b < n) {
         float o = 0.f;
 #pragma unroll
-        for (int r = 0; r < ROWS; ++r) {
-          const int d = p + LS_QUARTERS * r;
-          if (d < dim) {
-            s[r] = fmaf(as[b][d], s[r], ks[b][d] * v[b]);
-            if (MODE != 1) o = fmaf(s[r], qs[b][d], o);
+        for (int r = 0; r < ROWS; r += 4) {
+          // Four rows' staged values at once (rows beyond the head's channels hold what the batch
+          // before left or nothing: their state stays zero because their k is never staged: see below).
+          const ls_f32x4 a4 = *reinterpret_cast<const ls_f32x4*>(&as[b][p * ROWS + r]);
+          const ls_f32x4 k4 = *reinterpret_cast<const ls_f32x4*>(&ks[b][p * ROWS + r]);
+          ls_f32x4 q4 = ls_f32x4{0.f, 0.f, 0.f, 0.f};
+          if (MODE != 1) q4 = *reinterpret_cast<const ls_f32x4*>(&qs[b][p * ROWS + r]);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            s[r + e] = fmaf(a4[e], s[r + e], k4[e] * v[b]);
+            if (MODE != 1) o = fmaf(s[r + e], q4[e], o);
           }
         }
         if (MODE != 1) shares[b][p][c] = o;
@@ -160,7 +185,7 @@ linear_state_scan_kernel(float* __restrict__ out, const P* __restrict__ proj, in
   if (to && has_col) {
 #pragma unroll
     for (int r = 0; r < ROWS; ++r) {
-      const int d = p + LS_QUARTERS * r;
+      const int d = p * ROWS + r;
       if (d < dim) to[(size_t)d * vdim + col] = s[r];
     }
   }

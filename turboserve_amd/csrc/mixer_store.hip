@@ -15,10 +15,20 @@
 
 #include "common.hpp"
 
+// The sum of a projection's partial sums, added in split order, eight loads in flight at a time (a
+// loop of load, wait, add would cost a trip to memory per split).
 template <typename P>
 __device__ __forceinline__ float folded(const P* p, int splits, size_t stride) {
-  float s = to_float(p[0]);
-  for (int i = 1; i < splits; ++i) s += to_float(p[(size_t)i * stride]);
+  if (splits == 1) return to_float(p[0]);
+  float s = 0.f;
+  for (int first = 0; first < splits; first += 8) {
+    float v[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = to_float(p[(size_t)min(first + j, splits - 1) * stride]);
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      if (first + j < splits) s += v[j];
+  }
   return s;
 }
 

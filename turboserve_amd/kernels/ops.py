@@ -782,7 +782,7 @@ class Ops:
         _need(a2.shape == (heads * head_dim, low) and a2.dtype == dtype and a2.is_contiguous()
               and a2_bias.shape == (heads * head_dim,) and a2_bias.dtype == dtype and a2_bias.is_contiguous(),
               "a2 [H D, R] and its bias [H D] of the run dtype")
-        _need(head_dim <= 256 and low <= 64, "up to 256 key channels a head and a decay input of up to 64")
+        _need(head_dim <= 256 and low <= 128, "up to 256 key channels a head and a decay input of up to 128")
         _need(state.dtype == torch.float32 and state.is_contiguous() and tuple(state.shape[1:]) == (heads, head_dim, value_dim),
               "state must be contiguous float32 [slots, H, D, Dv]")
         _need(out.dtype == torch.float32 and out.is_contiguous() and out.shape == (tokens, heads * value_dim),

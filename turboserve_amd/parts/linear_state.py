@@ -52,8 +52,8 @@ class GatedLinearAttention(Mixer):
             raise ValueError(f"{prefix or 'gated linear attention'}: sizes and tau must be positive")
         if self.head_dim > 256 or self.num_heads > 65535:
             raise ValueError(f"{prefix or 'gated linear attention'}: the kernel takes up to 256 key channels a head")
-        if self.decay_rank is not None and not 1 <= self.decay_rank <= 64:
-            raise ValueError(f"{prefix or 'gated linear attention'}: a decay input of {self.decay_rank} is outside 1..64")
+        if self.decay_rank is not None and not 1 <= self.decay_rank <= 128:
+            raise ValueError(f"{prefix or 'gated linear attention'}: a decay input of {self.decay_rank} is outside 1..128")
         self.names = {"q": "q", "k": "k", "v": "v", "gate": "g", "o": "o", "norm": "norm", "a1": "a1", "a2": "a2",
                       "a2_bias": "a2.b", **(names or {})}
         self.key_size = self.num_heads * self.head_dim
@@ -91,9 +91,9 @@ class GatedLinearAttention(Mixer):
         n = self.names
         a1 = tensors[self.name(n["a1"])]
         self.a2 = tensors[self.name(n["a2"])].contiguous()
-        if a1.shape[0] != self.a2.shape[1] or not 1 <= a1.shape[0] <= 64:
+        if a1.shape[0] != self.a2.shape[1] or not 1 <= a1.shape[0] <= 128:
             raise ValueError(f"{self.prefix}: the decay's two matrices meet at {a1.shape[0]} and {self.a2.shape[1]} "
-                             "elements; they must agree and be 1..64")
+                             "elements; they must agree and be 1..128")
         self.low = int(a1.shape[0])
         self.fused = torch.cat([tensors[self.name(n[key])] for key in ("q", "k", "v", "gate")] + [a1], dim=0).contiguous()
         del a1
