@@ -189,6 +189,7 @@ def test_the_state_walk_whole_and_in_pieces(ops, heads, dim, vdim, low, lengths)
     (6, 2, 32, 32, False, 32, dict(chunk=64, sinks=1.0, slopes=True)),
     (16, 1, 80, 64, True, 16, dict()),
     (8, 1, 320, 256, True, 16, dict()),
+    (4, 1, 448, 384, True, 16, dict()),
     (70, 1, 40, 24, True, 8, dict(window=33)),
     (8, 4, 128, 128, False, 16, dict(chunk=1024, sinks=2.0, slopes=True, softcap=5.0)),
     (2, 2, 48, 104, False, 64, dict(window=100, sinks=0.5)),

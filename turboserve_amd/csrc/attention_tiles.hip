@@ -17,7 +17,7 @@
 // x 64 keys) = Q K^T by v_mfma_f32_16x16x32_bf16, online softmax in the accumulator layout, P
 // through LDS into the operand layout, O += P V.
 //
-// Sizes: Dk (up to 384) and Dv (up to 256) multiples of 8; pages of 8 tokens or more (a multiple of 8).
+// Sizes: Dk (up to 384; 448 with the values inside the key rows) and Dv (up to 256; 384) multiples of 8; pages of 8 tokens or more (a multiple of 8).
 #include "common.hpp"
 
 typedef __bf16 fa_bf16x8 __attribute__((ext_vector_type(8)));
@@ -413,9 +413,10 @@ extern "C" int ts_attention_tiles(void* out, void* partial_o, void* partial_ml, 
   if (mode == 1 && splits > 1 && (!partial_o || !partial_ml)) return TS_ERR_ARG;
   if (mode < 0 || mode > 1 || splits < 1 || splits > 65535) return TS_ERR_ARG;
   if (heads < 1 || kv_heads < 1 || heads % kv_heads != 0 || heads > 65535) return TS_ERR_SHAPE;
-  if (dk < 8 || dk > 384 || dk % 8 != 0 || dv < 8 || dv > 256 || dv % 8 != 0 || block_size < 8 || block_size % 8 != 0)
+  if (dk < 8 || dk > 448 || dk % 8 != 0 || dv < 8 || dv > 384 || dv % 8 != 0 || block_size < 8 || block_size % 8 != 0)
     return TS_ERR_SHAPE;
   if (!v_pages && dv > dk) return TS_ERR_SHAPE;
+  if (v_pages && (dk > 384 || dv > 256)) return TS_ERR_SHAPE;  // the widest tiles are built for values inside the key rows
   if ((((uintptr_t)q | (uintptr_t)k_pages | (uintptr_t)v_pages) & 15) != 0 || (q_stride % 8) != 0) return TS_ERR_ARG;
   const FaRule rule = {scale, softcap, sinks, window, chunk};
   const int group_heads = heads / kv_heads;
@@ -431,6 +432,7 @@ extern "C" int ts_attention_tiles(void* out, void* partial_o, void* partial_ml, 
   if (kd <= 4 && vd <= 8) FA_SIZE(4, 8);
   if (kd <= 8 && vd <= 16) FA_SIZE(8, 16);
   if (kd <= 12 && vd <= 16) FA_SIZE(12, 16);
+  if (kd <= 14 && vd <= 24) FA_SIZE(14, 24);
 #undef FA_SIZE
   return TS_ERR_SHAPE;
 }

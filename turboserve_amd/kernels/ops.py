@@ -1068,12 +1068,15 @@ class Ops:
         return out
 
     @staticmethod
-    def tiled_attention_supported(dtype: torch.dtype, head_dim: int, value_dim: int, block_size: int, q_stride: int) -> bool:
+    def tiled_attention_supported(dtype: torch.dtype, head_dim: int, value_dim: int, block_size: int, q_stride: int,
+                                  values_in_keys: bool = False) -> bool:
         """Whether :meth:`attention_tiles` takes this geometry: bfloat16, key rows of up to 384 and
-        values of up to 256 elements, both multiples of 8 (16-byte accesses), pages of a multiple of 8
-        tokens, query rows 16 bytes apart or a multiple of that."""
-        return (dtype == torch.bfloat16 and head_dim % 8 == 0 and 8 <= head_dim <= 384 and value_dim % 8 == 0
-                and 8 <= value_dim <= 256 and block_size % 8 == 0 and q_stride % 8 == 0)
+        values of up to 256 elements (448 and 384 where the values lie inside the key rows), both
+        multiples of 8 (16-byte accesses), pages of a multiple of 8 tokens, query rows 16 bytes apart
+        or a multiple of that."""
+        widest = (448, 384) if values_in_keys else (384, 256)
+        return (dtype == torch.bfloat16 and head_dim % 8 == 0 and 8 <= head_dim <= widest[0] and value_dim % 8 == 0
+                and 8 <= value_dim <= widest[1] and block_size % 8 == 0 and q_stride % 8 == 0)
 
     @staticmethod
     def attention_tile_list(query_lens, rows: int = 64) -> list[list[int]]:
@@ -1109,7 +1112,8 @@ class Ops:
             _check_pages(k_pages, v_pages, q.dtype, any_value_width=True)
             value_dim = v_pages.shape[2]
         _need(value_dim is not None and (v_pages is not None or value_dim <= head_dim), "values inside the keys are their first value_dim elements")
-        _need(self.tiled_attention_supported(q.dtype, head_dim, value_dim, block_size, q_stride), "a geometry the tiled attention kernel does not take")
+        _need(self.tiled_attention_supported(q.dtype, head_dim, value_dim, block_size, q_stride, v_pages is None),
+              "a geometry the tiled attention kernel does not take")
         _need(heads % kv_heads == 0 and q.is_contiguous() and q.numel() >= tokens * q_stride and q_stride >= heads * head_dim,
               "q does not hold [T, q_stride] rows of the heads")
         _need(block_table.dim() == 2 and query_start_loc.numel() >= num_prefill_seqs + num_decode_seqs + 1, "block_table [S, MB], row ranges [S + 1]")

@@ -113,7 +113,7 @@ class LatentAttention(Mixer):
         carried = ops.per_head_rows(q_plain, self.up_k)
         q_wide[:, :, : self.rank].copy_(carried.view(tokens, self.num_heads, self.rank))
         stride = self.num_heads * self.wide
-        if ops.tiled_attention_supported(dtype, self.wide, self.rank, cache.block_size, stride):
+        if ops.tiled_attention_supported(dtype, self.wide, self.rank, cache.block_size, stride, True):
             attended = tiled_attention(ops, q_wide.view(tokens, stride), stride, cache.k, None, ctx.block_tables[cache.group],
                                        ctx, heads=self.num_heads, scale=self.scale, value_dim=self.rank)
         else:
