@@ -285,3 +285,34 @@ def test_manager_tables_report_released_pages():
     assert held.tables[1][0] == PAD_PAGE and PAD_PAGE not in held.tables[0]
     manager.free("r")
     manager.check_invariants()
+
+
+def test_pages_below_the_current_chunk_are_given_back():
+    """A group whose tokens read only their own chunk of positions holds the pages of the chunk that
+    the next token lies in, and of the portion being written; everything below goes back."""
+    manager = CacheManager([None], 6, 4, 1, chunks=[8])
+    manager.admit("a")
+    manager.append("a", 7)                       # positions 0..6: chunk 0, pages 0 and 1
+    assert manager.get("a").released == [0]
+    manager.append("a", 3)                       # the portion starts at 7, still chunk 0: nothing goes back
+    assert manager.get("a").released == [0] and manager.pools[0].num_in_use == 3
+    manager.append("a", 1)                       # starts at 10, chunk 1 begins at 8: pages 0 and 1 go back
+    entry = manager.get("a")
+    assert entry.released == [2] and list(entry.tables[0])[:2] == [-1, -1] and manager.pools[0].num_in_use == 1
+    manager.check_invariants()
+    for _ in range(40):                          # 40 more tokens on a pool of 6 pages: only by giving pages back
+        manager.append("a", 1)
+    assert manager.pools[0].num_in_use <= 3
+    manager.check_invariants()
+    # The peak a request needs is what a chunk and a portion span, not its length.
+    assert manager.peak_pages(0, 10_000, 5) == 4 and manager.fits_pool(10_000, 5)
+    # A window and chunks together: whichever bound is higher.
+    both = CacheManager([6], 8, 4, 1, chunks=[16])
+    both.admit("b")
+    both.append("b", 15)
+    both.append("b", 1)                          # starts at 15: window from 10, chunk 0 from 0 -> pages 0, 1 go back
+    assert both.get("b").released == [2]
+    both.append("b", 1)                          # starts at 16: chunk 1 begins at 16 -> pages 0..3 go back
+    assert both.get("b").released == [4]
+    manager.free("a")
+    both.free("b")

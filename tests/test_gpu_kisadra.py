@@ -266,6 +266,22 @@ def test_one_layer_models(tmp_path, which, dtype, looped):
             assert excess(got[rid], want[rid], dtype) <= 1.0, (which, rid)
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_chunked_layer_on_a_pool_smaller_than_the_request(tmp_path, dtype):
+    """Layers that read only their own chunk give the pages below it back while the request runs: 150
+    tokens go through a pool of 64, in portions and token by token, and every position is still right."""
+    chunked = kt.layer(kt.attention(4, 2, 16, 16, 16, scale=0.4), kt.dense(44))
+    config = {"architecture": "Kisadra", "vocab": 61, "width": 40, "norm": {"eps": 1e-5}, "layers": [chunked, chunked],
+              "loop": {"start": 0, "stop": 1, "times": 2}}
+    stored = torch.float32 if dtype == "float32" else torch.bfloat16
+    folder = kt.make_model_dir(tmp_path / "m", config, 77, stored, std=0.2 if dtype == "float32" else 0.1)
+    requests = {"long": tokens_of(61, 150, 9)}
+    want = kt.plain_logits(folder, requests["long"])
+    for steps in (th.portions(requests, (20, 3, 11, 2)), th.prefix_then_single(requests, tail=130)):
+        got = th.collect(steps, run_trace(folder, dtype, 8, steps, max_tokens=64), requests)["long"]
+        assert excess(got, want, dtype) <= 1.0
+
+
 # ---------------------------------------------------------------------------------------------
 # whole models, every cutting
 # ---------------------------------------------------------------------------------------------

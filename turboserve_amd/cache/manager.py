@@ -3,7 +3,7 @@
 One page pool and one block table per request *for each group* of layers.  A request's pages
 are taken portion by portion as its tokens are scheduled (the reference's ``append_slots``,
 src/turboserve/engine/core/block_manager.py:222-246) and given back when it finishes, is
-preempted, or, in a windowed group, when every later query's window has passed them.  A slot
+preempted, or, in a group with a window or chunks, when no later query can read them.  A slot
 is ``page * page_size + offset`` (block_manager.py:248-268).  Released entries of a block
 table hold ``PAD_PAGE``; no kernel reads below a window's lower bound.
 """
@@ -25,6 +25,17 @@ def ceil_div(a: int, b: int) -> int:
     return -(-a // b)
 
 
+def lowest_key_read(position: int, window: int | None, chunk: int | None) -> int:
+    """The lowest key a query at ``position`` or later reads: ``position - window + 1`` under a window,
+    the first position of the query's chunk under chunks, the larger of the two under both, else 0."""
+    lowest = 0
+    if window is not None:
+        lowest = max(lowest, position - window + 1)
+    if chunk is not None:
+        lowest = max(lowest, (position // chunk) * chunk)
+    return lowest
+
+
 @dataclass
 class RequestCache:
     """What one request holds."""
@@ -43,6 +54,7 @@ class CacheManager:
         num_pages: Sequence[int] | int,
         page_size: int,
         num_state_slots: int,
+        chunks: Sequence[int | None] | None = None,
     ) -> None:
         if page_size < 1 or page_size & (page_size - 1):
             raise ValueError(f"page_size must be a power of two, got {page_size}")
@@ -50,6 +62,10 @@ class CacheManager:
         if len(counts) != len(windows):
             raise ValueError(f"{len(counts)} pool sizes for {len(windows)} groups")
         self.windows = list(windows)
+        #: Per group: a token reads no key below its own chunk of this many positions (``None``: no chunks).
+        self.chunks = [None] * len(self.windows) if chunks is None else list(chunks)
+        if len(self.chunks) != len(self.windows):
+            raise ValueError(f"{len(self.chunks)} chunk sizes for {len(self.windows)} groups")
         self.page_size = page_size
         self.pools = [PageAllocator(n, page_size) for n in counts]
         self.state_slots = StateSlotPool(num_state_slots)
@@ -75,10 +91,12 @@ class CacheManager:
         portions are at most ``max_portion`` tokens: all of them, or what a window plus one
         portion spans (one more for the window's start inside a page)."""
         pages = ceil_div(total_tokens, self.page_size)
-        window = self.windows[group]
-        if window is None:
+        # A chunk of C positions bounds what is read like a window of C: the first token of a
+        # portion reads no further back than C - 1 keys.
+        reach = [r for r in (self.windows[group], self.chunks[group]) if r is not None]
+        if not reach:
             return pages
-        return min(pages, ceil_div(window - 1 + max_portion, self.page_size) + 1)
+        return min(pages, ceil_div(min(reach) - 1 + max_portion, self.page_size) + 1)
 
     def fits_pool(self, total_tokens: int, max_portion: int) -> bool:
         """Whether the request could run if it had the pools to itself."""
@@ -113,11 +131,7 @@ class CacheManager:
 
     def _releasable(self, entry: RequestCache, group: int, start: int) -> int:
         """Leading logical pages no query at position ``>= start`` can see."""
-        window = self.windows[group]
-        if window is None:
-            return 0
-        lowest_key = max(0, start - window + 1)
-        return min(lowest_key // self.page_size, len(entry.tables[group]))
+        return min(lowest_key_read(start, self.windows[group], self.chunks[group]) // self.page_size, len(entry.tables[group]))
 
     def pages_short(self, request: Hashable, num_new: int) -> list[int]:
         """Per group, how many pages more than are free a portion of ``num_new`` tokens needs

@@ -243,16 +243,22 @@ attention_tiles_kernel(uint16_t* __restrict__ out, float* __restrict__ partial_o
     fa_f32x4 s[4];
 #pragma unroll
     for (int ct = 0; ct < 4; ++ct) s[ct] = fa_f32x4{0.f, 0.f, 0.f, 0.f};
+    // (Every piece of the size class is multiplied, also those past Dk, which hold zeros: a test
+    // per piece would cut this stretch into pieces that each wait for their own LDS reads.)
 #pragma unroll
     for (int kd = 0; kd < KD; ++kd) {
-      if (32 * kd < dk) {
 #pragma unroll
-        for (int ct = 0; ct < 4; ++ct) {
-          const ts_u32x4 kf = *reinterpret_cast<const ts_u32x4*>(ks + (16 * ct + r16) * K_ROW + 32 * kd + 8 * group);
-          s[ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(fa_bf16x8, qf[kd]),
-                                                          __builtin_bit_cast(fa_bf16x8, kf), s[ct], 0, 0, 0);
-        }
+      for (int ct = 0; ct < 4; ++ct) {
+        const ts_u32x4 kf = *reinterpret_cast<const ts_u32x4*>(ks + (16 * ct + r16) * K_ROW + 32 * kd + 8 * group);
+        s[ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(fa_bf16x8, qf[kd]),
+                                                        __builtin_bit_cast(fa_bf16x8, kf), s[ct], 0, 0, 0);
       }
+    }
+    if (rule.softcap > 0.f) {
+#pragma unroll
+      for (int ct = 0; ct < 4; ++ct)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) s[ct][i] = rule.softcap / rule.scale * tanhf(s[ct][i] * rule.scale / rule.softcap);
     }
     // Scores of this lane: row 4 group + i, key key0 + 16 ct + r16.
     float tile_max[4];
@@ -263,9 +269,7 @@ attention_tiles_kernel(uint16_t* __restrict__ out, float* __restrict__ partial_o
       const int key = key0 + 16 * ct + r16;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        float v = s[ct][i] * rule.scale;
-        if (rule.softcap > 0.f) v = rule.softcap * tanhf(v / rule.softcap);
-        v = fmaf(slope[i], (float)(key - pos[i]), v);
+        float v = fmaf(slope[i], (float)(key - pos[i]), s[ct][i] * rule.scale);
         v = (key >= low[i] && key <= pos[i]) ? v : -INFINITY;
         s[ct][i] = v;
         tile_max[i] = fmaxf(tile_max[i], v);
@@ -308,11 +312,9 @@ attention_tiles_kernel(uint16_t* __restrict__ out, float* __restrict__ partial_o
       const ts_u32x4 pf = *reinterpret_cast<const ts_u32x4*>(my_p + r16 * P_ROW + 32 * kk + 8 * group);
 #pragma unroll
       for (int vt = 0; vt < VD; ++vt) {
-        if (16 * vt < dv) {
-          const ts_u32x4 vf = *reinterpret_cast<const ts_u32x4*>(vs + (16 * vt + r16) * V_ROW + 32 * kk + 8 * group);
-          o[vt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(fa_bf16x8, pf),
-                                                          __builtin_bit_cast(fa_bf16x8, vf), o[vt], 0, 0, 0);
-        }
+        const ts_u32x4 vf = *reinterpret_cast<const ts_u32x4*>(vs + (16 * vt + r16) * V_ROW + 32 * kk + 8 * group);
+        o[vt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(fa_bf16x8, pf),
+                                                        __builtin_bit_cast(fa_bf16x8, vf), o[vt], 0, 0, 0);
       }
     }
   }
@@ -430,7 +432,10 @@ extern "C" int ts_attention_tiles(void* out, void* partial_o, void* partial_ml, 
                               dk, dv, block_size, slopes, rule, splits)
   if (kd <= 2 && vd <= 4) FA_SIZE(2, 4);
   if (kd <= 4 && vd <= 8) FA_SIZE(4, 8);
+  if (kd <= 4 && vd <= 16) FA_SIZE(4, 16);
+  if (kd <= 8 && vd <= 8) FA_SIZE(8, 8);
   if (kd <= 8 && vd <= 16) FA_SIZE(8, 16);
+  if (kd <= 10 && vd <= 16) FA_SIZE(10, 16);
   if (kd <= 12 && vd <= 16) FA_SIZE(12, 16);
   if (kd <= 14 && vd <= 24) FA_SIZE(14, 24);
 #undef FA_SIZE

@@ -48,6 +48,7 @@ class StepLimits:
 
     num_pages: Sequence[int]
     windows: Sequence[int | None]
+    chunks: Sequence[int | None] | None = None  # per group: a token reads no key below its own chunk
     vocab_size: int | None = None
     num_state_slots: int | None = None  # slots 0 .. num_state_slots are valid (the last is the padding row)
 
@@ -280,6 +281,9 @@ def check_packed(data: np.ndarray, layout: StepLayout, entries: Sequence[StepEnt
                                  f"{len(entry.tables[group])} pages, {int(contexts[row])} tokens need "
                                  f"{-(-int(contexts[row]) // page_size)}")
         lowest_key = np.zeros(seqs, dtype=np.int64) if window is None else np.maximum(0, first_position - window + 1)
+        chunk = None if limits.chunks is None else limits.chunks[group]
+        if chunk is not None:
+            lowest_key = np.maximum(lowest_key, (np.maximum(first_position, 0) // chunk) * chunk)
         columns = np.arange(width, dtype=np.int64)[None, :]
         read = (columns >= (lowest_key // page_size)[:, None]) & (columns < (-(-contexts // page_size))[:, None])
         missing = np.argwhere(read & (table < 0))

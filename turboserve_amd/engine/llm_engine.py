@@ -124,7 +124,8 @@ class LLMEngine:
         if scheduler is None:
             if storage is None:
                 raise ValueError("an engine built around a stand-in runner needs its scheduler passed in")
-            cache = CacheManager(storage.layout.windows(), storage.num_pages, sched_cfg.block_size, sched_cfg.max_num_seqs)
+            cache = CacheManager(storage.layout.windows(), storage.num_pages, sched_cfg.block_size, sched_cfg.max_num_seqs,
+                                 chunks=storage.layout.chunks())
             scheduler = Scheduler(sched_cfg, cache)
         self.scheduler = scheduler
         self.runner = runner if runner is not None else ModelRunner(model, storage)

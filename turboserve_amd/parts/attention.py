@@ -118,7 +118,7 @@ class GroupedQueryAttention(Mixer):
 
     def cache_need(self) -> CacheNeed:
         return PagedKV(self.num_kv_heads, self.head_dim, self.window,
-                       None if self.value_dim == self.head_dim else self.value_dim)
+                       None if self.value_dim == self.head_dim else self.value_dim, self.chunk)
 
     def is_capturable(self) -> bool:
         return self.capturable and self.position.is_capturable()

@@ -55,12 +55,15 @@ class PagedKV:
     """A mixer's need for per-token cache pages: per token ``num_kv_heads`` keys of ``head_dim``
     elements and as many values of ``value_dim`` (``None``: as wide as the keys; 0: the mixer
     caches one vector per token and head, and the value pages have no room at all);
-    ``window`` keys are ever read again (``None``: all of them)."""
+    ``window`` keys are ever read again (``None``: all of them); with ``chunk = C`` a token at
+    position ``p`` reads no key below ``(p // C) * C``, so pages below the chunk of the next token are
+    never read again either."""
 
     num_kv_heads: int
     head_dim: int
     window: int | None = None
     value_dim: int | None = None
+    chunk: int | None = None
 
     @property
     def value_width(self) -> int:
