@@ -345,27 +345,35 @@ attention_tiles_kernel(uint16_t* __restrict__ out, float* __restrict__ partial_o
   }
 }
 
-// out[request's token, head, :] from the shares of its keys: one block per (request, head).
+// out[request's token, head, :] from the shares of its keys: one block per (request, head).  The
+// shares' maxima and sums are fetched side by side (one thread each) and turned into weights in LDS.
+#define FA_MAX_SPLITS 64
 __global__ void __launch_bounds__(128)
 attention_tiles_combine_kernel(uint16_t* __restrict__ out, const float* __restrict__ partial_o,
                                const float* __restrict__ partial_ml, const int* __restrict__ query_start_loc,
                                int first_seq, int heads, int dv, int splits, float sinks) {
+  __shared__ float weight[FA_MAX_SPLITS];
+  __shared__ float scratch[16];
   const int item = blockIdx.x, h = blockIdx.y;
   const size_t base = ((size_t)item * heads + h) * splits;
-  float m = sinks > 0.f ? 0.f : -INFINITY;
-  for (int sp = 0; sp < splits; ++sp) m = fmaxf(m, partial_ml[2 * (base + sp)]);
-  float l = sinks > 0.f ? sinks * expf(0.f - m) : 0.f;
-  for (int sp = 0; sp < splits; ++sp) {
-    const float ms = partial_ml[2 * (base + sp)];
-    if (ms != -INFINITY) l += partial_ml[2 * (base + sp) + 1] * expf(ms - m);
-  }
+  const int sp = threadIdx.x;
+  const float ms = sp < splits ? partial_ml[2 * (base + sp)] : -INFINITY;
+  const float ls = sp < splits ? partial_ml[2 * (base + sp) + 1] : 0.f;
+  const float m = fmaxf(block_max(ms, scratch), sinks > 0.f ? 0.f : -INFINITY);
+  const float w = ms == -INFINITY ? 0.f : expf(ms - m);
+  if (sp < splits) weight[sp] = w;
+  const float l = block_sum(ls * w, scratch) + (sinks > 0.f ? sinks * expf(0.f - m) : 0.f);  // (its barriers publish the weights)
   const float inv = l > 0.f ? 1.f / l : 0.f;
   const int row = query_start_loc[first_seq + item];
   for (int d = threadIdx.x; d < dv; d += blockDim.x) {
     float acc = 0.f;
-    for (int sp = 0; sp < splits; ++sp) {
-      const float ms = partial_ml[2 * (base + sp)];
-      if (ms != -INFINITY) acc = fmaf(partial_o[(base + sp) * dv + d], expf(ms - m), acc);
+    for (int first = 0; first < splits; first += 8) {  // eight loads in flight
+      float v[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) v[j] = partial_o[(base + min(first + j, splits - 1)) * dv + d];
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        if (first + j < splits) acc = fmaf(v[j], weight[first + j], acc);
     }
     out[((size_t)row * heads + h) * dv + d] = from_float<bf16_t>(acc * inv).bits;
   }
@@ -413,7 +421,7 @@ extern "C" int ts_attention_tiles(void* out, void* partial_o, void* partial_ml, 
   if (!out || !q || !k_pages || !block_table || !query_start_loc || !context_lens) return TS_ERR_ARG;
   if (mode == 0 && (!tiles || splits != 1)) return TS_ERR_ARG;
   if (mode == 1 && splits > 1 && (!partial_o || !partial_ml)) return TS_ERR_ARG;
-  if (mode < 0 || mode > 1 || splits < 1 || splits > 65535) return TS_ERR_ARG;
+  if (mode < 0 || mode > 1 || splits < 1 || splits > FA_MAX_SPLITS) return TS_ERR_ARG;
   if (heads < 1 || kv_heads < 1 || heads % kv_heads != 0 || heads > 65535) return TS_ERR_SHAPE;
   if (dk < 8 || dk > 448 || dk % 8 != 0 || dv < 8 || dv > 384 || dv % 8 != 0 || block_size < 8 || block_size % 8 != 0)
     return TS_ERR_SHAPE;
@@ -446,7 +454,7 @@ extern "C" int ts_attention_tiles_combine(void* out, const void* partial_o, cons
                                           const int* query_start_loc, int items, int first_seq, int heads, int dv,
                                           int splits, float sinks, hipStream_t stream) {
   if (items == 0) return TS_OK;
-  if (!out || !partial_o || !partial_ml || !query_start_loc || splits < 1 || heads < 1 || heads > 65535 || dv < 1)
+  if (!out || !partial_o || !partial_ml || !query_start_loc || splits < 1 || splits > FA_MAX_SPLITS || heads < 1 || heads > 65535 || dv < 1)
     return TS_ERR_ARG;
   hipLaunchKernelGGL(attention_tiles_combine_kernel, dim3(items, heads), dim3(128), 0, stream, (uint16_t*)out,
                      (const float*)partial_o, (const float*)partial_ml, query_start_loc, first_seq, heads, dv, splits, sinks);

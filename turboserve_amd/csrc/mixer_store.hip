@@ -38,7 +38,7 @@ __device__ __forceinline__ float folded(const P* p, int splits, size_t stride) {
 // likewise over their Hkv D.  Keys go to [NB, Hkv, BS, D], values to the transposed [NB, Hkv, Dv, BS].
 // ---------------------------------------------------------------------------------------------
 template <typename T, typename P>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(1024)
 span_norm_store_kernel(T* q_out, long q_stride, const P* proj, int splits, size_t split_stride,
                        T* __restrict__ k_pages, T* __restrict__ v_pages, const T* __restrict__ q_gain,
                        const T* __restrict__ k_gain, float eps, float gain_offset, const int* __restrict__ slots,
@@ -86,7 +86,8 @@ static int span_norm_store_launch(void* q_out, long q_stride, const void* proj, 
                                   void* k_pages, void* v_pages, const void* q_gain, const void* k_gain, float eps,
                                   float gain_offset, const int* slots, int tokens, int heads, int kv_heads, int dim,
                                   int vdim, int block_size, hipStream_t stream) {
-  hipLaunchKernelGGL((span_norm_store_kernel<T, P>), dim3(tokens), dim3(256), 0, stream, (T*)q_out, q_stride,
+  // A step of few tokens has few blocks: each then takes a whole compute unit's threads.
+  hipLaunchKernelGGL((span_norm_store_kernel<T, P>), dim3(tokens), dim3(tokens <= 64 ? 1024 : 256), 0, stream, (T*)q_out, q_stride,
                      (const P*)proj, splits, (size_t)split_stride, (T*)k_pages, (T*)v_pages, (const T*)q_gain,
                      (const T*)k_gain, eps, gain_offset, slots, heads, kv_heads, dim, vdim, block_size);
   return ts_launch_status();
@@ -129,7 +130,7 @@ __device__ __forceinline__ float turned_element(const float* part, int i, int tu
 }
 
 template <typename T, typename P>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(1024)
 latent_store_kernel(T* __restrict__ q_plain, T* __restrict__ q_wide, const P* proj, int splits, size_t split_stride,
                     T* __restrict__ k_pages, const T* __restrict__ gain, float eps,
                     const float* __restrict__ cos_table, const float* __restrict__ sin_table,
@@ -182,7 +183,7 @@ static int latent_store_launch(void* q_plain, void* q_wide, const void* proj, in
                                int turned, int block_size, hipStream_t stream) {
   const size_t lds = (size_t)(heads * rot + rot + rank) * sizeof(float);
   if (lds > 60 * 1024) return TS_ERR_SHAPE;
-  hipLaunchKernelGGL((latent_store_kernel<T, P>), dim3(tokens), dim3(256), lds, stream, (T*)q_plain, (T*)q_wide,
+  hipLaunchKernelGGL((latent_store_kernel<T, P>), dim3(tokens), dim3(tokens <= 64 ? 1024 : 256), lds, stream, (T*)q_plain, (T*)q_wide,
                      (const P*)proj, splits, (size_t)split_stride, (T*)k_pages, (const T*)gain, eps, cos_table, sin_table,
                      positions, slots, heads, dim, rot, rank, turned, block_size);
   return ts_launch_status();
