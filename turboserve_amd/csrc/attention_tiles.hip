@@ -93,10 +93,12 @@ attention_tiles_kernel(uint16_t* __restrict__ out, float* __restrict__ partial_o
     tile_rows = min(FA_ROWS, kvh * group_heads + group_heads - head_first);
     tile_first_row = query_start_loc[seq];
   } else {
-    seq = tiles[2 * blockIdx.x];
-    tile_first_row = tiles[2 * blockIdx.x + 1];
+    // Heads are the fast index of the grid, so workgroups start in the order of the tile list: the
+    // host puts the tiles with the most keys first.
+    seq = tiles[2 * blockIdx.y];
+    tile_first_row = tiles[2 * blockIdx.y + 1];
     tile_rows = min(FA_ROWS, query_start_loc[seq + 1] - tile_first_row);
-    head_first = blockIdx.y;
+    head_first = blockIdx.x;
     kvh = head_first / group_heads;
   }
   const int context = context_lens[seq];
@@ -408,7 +410,7 @@ static int tiles_launch(bool single, bool values_in_keys, dim3 grid, hipStream_t
   return ts_launch_status();
 }
 
-// mode 0: prompt portions, `items` tiles (pairs: request, first row) and grid.y = heads;
+// mode 0: prompt portions, `items` tiles (pairs: request, first row), each for every head;
 // mode 1: `items` requests of one token each from `first_seq` on, their keys shared out over `splits`.
 // out [T, heads, Dv] bfloat16.  v_pages null: the values are the keys' first Dv elements.
 extern "C" int ts_attention_tiles(void* out, void* partial_o, void* partial_ml, const void* q, long q_stride,
@@ -430,7 +432,8 @@ extern "C" int ts_attention_tiles(void* out, void* partial_o, void* partial_ml, 
   if ((((uintptr_t)q | (uintptr_t)k_pages | (uintptr_t)v_pages) & 15) != 0 || (q_stride % 8) != 0) return TS_ERR_ARG;
   const FaRule rule = {scale, softcap, sinks, window, chunk};
   const int group_heads = heads / kv_heads;
-  const dim3 grid(items, mode == 0 ? heads : kv_heads * ((group_heads + FA_ROWS - 1) / FA_ROWS), splits);
+  if (mode == 0 && items > 65535) return TS_ERR_SHAPE;
+  const dim3 grid = mode == 0 ? dim3(heads, items, 1) : dim3(items, kv_heads * ((group_heads + FA_ROWS - 1) / FA_ROWS), splits);
   const bool single = mode == 1, in_keys = v_pages == nullptr;
   const int kd = (dk + 31) / 32, vd = (dv + 15) / 16;
 #define FA_SIZE(KD, VD)                                                                                                 \

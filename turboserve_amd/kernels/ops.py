@@ -1079,14 +1079,23 @@ class Ops:
                 and 8 <= value_dim <= widest[1] and block_size % 8 == 0 and q_stride % 8 == 0)
 
     @staticmethod
-    def attention_tile_list(query_lens, rows: int = 64) -> list[list[int]]:
+    def attention_tile_list(query_lens, context_lens=None, rows: int = 64, *, window: int | None = None,
+                            chunk: int | None = None) -> list[list[int]]:
         """``[request, first row]`` of every tile of ``rows`` consecutive tokens of the requests
-        ``0 .. len(query_lens) - 1`` at the front of a step."""
+        ``0 .. len(query_lens) - 1`` at the front of a step; with the requests' ``context_lens``, the
+        tiles that see the most keys (under the layer's ``window`` and ``chunk``) come first, so that
+        the longest walks start first."""
         tiles, row = [], 0
         for request, count in enumerate(query_lens):
-            tiles.extend([request, row + first] for first in range(0, count, rows))
+            start = 0 if context_lens is None else context_lens[request] - count
+            for first in range(0, count, rows):
+                lowest = start + first
+                lowest = max(0 if window is None else lowest - window + 1, 0 if chunk is None else (lowest // chunk) * chunk)
+                tiles.append((start + first + min(rows, count - first) - lowest, request, row + first))
             row += count
-        return tiles
+        if context_lens is not None:
+            tiles.sort(key=lambda tile: -tile[0])
+        return [[request, first] for _, request, first in tiles]
 
     def attention_tiles(self, q: torch.Tensor, q_stride: int, k_pages: torch.Tensor, v_pages: torch.Tensor | None,
                         block_table: torch.Tensor, query_start_loc: torch.Tensor, context_lens: torch.Tensor, *,

@@ -17,8 +17,10 @@ def tiled_attention(ops, q, q_stride, k_pages, v_pages, table, ctx, **rule) -> t
     tokens is made once per step and shared by the layers (a recorded step has none: single tokens)."""
     tiles = None
     if ctx.num_prefill_seqs > 0:
-        tiles = ctx.derive("attention_tiles_64", lambda step: torch.tensor(
-            ops.attention_tile_list(step.query_lens[:step.num_prefill_seqs]), dtype=torch.int32, device=q.device))
+        reach = (rule.get("window"), rule.get("chunk"))
+        tiles = ctx.derive(("attention_tiles_64", *reach), lambda step: torch.tensor(
+            ops.attention_tile_list(step.query_lens[:step.num_prefill_seqs], step.context_lens_host[:step.num_prefill_seqs],
+                                    window=reach[0], chunk=reach[1]), dtype=torch.int32, device=q.device))
     return ops.attention_tiles(
         q, q_stride, k_pages, v_pages, table, ctx.query_start_loc, ctx.context_lens, tokens=ctx.num_tokens,
         prefill_tiles=tiles, num_prefill_seqs=ctx.num_prefill_seqs, num_decode_seqs=ctx.num_decode_seqs,
