@@ -115,6 +115,7 @@ linear_state_scan_kernel(float* __restrict__ out, const P* __restrict__ proj, in
     (&ks[0][0])[i] = 0.f;
     (&as[0][0])[i] = 0.f;
   }
+  for (int i = tid; i < LS_BATCH * LS_MAX_LOW; i += blockDim.x) (&ys[0][0])[i] = 0.f;  // (rows of a short batch are multiplied too)
 
   for (int base = 0; base < count; base += LS_BATCH) {
     const int n = min(LS_BATCH, count - base);
@@ -133,13 +134,30 @@ linear_state_scan_kernel(float* __restrict__ out, const P* __restrict__ proj, in
     if (tid < dim) {
       const T* w = a2 + ((size_t)h * dim + tid) * low;
       const float bias = to_float(a2_bias[(size_t)h * dim + tid]);
-      for (int b = 0; b < n; ++b) {
-        float z = bias;
-        for (int j = 0; j < low; ++j) z = fmaf(to_float(w[j]), ys[b][j], z);
-        // log sigmoid(z) = min(z, 0) - log(1 + exp(-|z|)); the decay is exp of it over tau.
-        const float a = expf((fminf(z, 0.f) - log1pf(expf(-fabsf(z)))) * inv_tau);
-        as[b][tid] = a;
-        if (MODE == 1) decay_product *= a;
+      // The channel's row of A2 is read once per batch, eight elements in flight at a time (read
+      // inside the loop over tokens it cost a trip to the caches per token and element).
+      float z[LS_BATCH];
+#pragma unroll
+      for (int b = 0; b < LS_BATCH; ++b) z[b] = bias;
+      for (int j0 = 0; j0 < low; j0 += 8) {
+        float wv[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) wv[u] = j0 + u < low ? to_float(w[j0 + u]) : 0.f;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const int j = min(j0 + u, low - 1);  // past the end: weight 0 on a value that is there
+#pragma unroll
+          for (int b = 0; b < LS_BATCH; ++b) z[b] = fmaf(wv[u], ys[b][j], z[b]);
+        }
+      }
+#pragma unroll
+      for (int b = 0; b < LS_BATCH; ++b) {
+        if (b < n) {
+          // log sigmoid(z) = min(z, 0) - log(1 + exp(-|z|)); the decay is exp of it over tau.
+          const float a = expf((fminf(z[b], 0.f) - log1pf(expf(-fabsf(z[b])))) * inv_tau);
+          as[b][tid] = a;
+          if (MODE == 1) decay_product *= a;
+        }
       }
     }
     __syncthreads();
