@@ -193,6 +193,10 @@ def test_the_state_walk_whole_and_in_pieces(ops, heads, dim, vdim, low, lengths)
     (70, 1, 40, 24, True, 8, dict(window=33)),
     (8, 4, 128, 128, False, 16, dict(chunk=1024, sinks=2.0, slopes=True, softcap=5.0)),
     (2, 2, 48, 104, False, 64, dict(window=100, sinks=0.5)),
+    (2, 1, 64, 256, False, 16, dict(chunk=300)),
+    (3, 3, 256, 128, False, 16, dict(sinks=1.0, slopes=True)),
+    (2, 1, 256, 256, True, 32, dict(chunk=77)),
+    (2, 2, 384, 200, False, 8, dict(slopes=True)),
 ])
 def test_the_tiled_attention_kernel_against_the_generic_one(ops, heads, kv_heads, dim, vdim, in_keys, page, rule):
     """bfloat16 on the matrix cores against the one-wavefront-per-row kernel on the same pages: prompt
