@@ -348,6 +348,13 @@ class Ops:
         #: Wavefronts (16 weight rows x one range of K each) the resident product aims for: 16 per compute unit.
         self.skinny_resident_waves = 16 * self.compute_units
 
+    def device_ints(self, values) -> torch.Tensor:
+        """A list (or nested list) of integers as an int32 tensor on the device, copied from pinned
+        memory behind the work already launched: a copy from pageable memory would make the host
+        wait until the stream has drained, and the device then waits for the host in turn."""
+        host = torch.tensor(values, dtype=torch.int32).pin_memory()
+        return host.to(self.device, non_blocking=True)
+
     def stream(self) -> int:
         """The handle of torch's current stream on this device (what every launch goes to)."""
         if self._raw_stream is not None:

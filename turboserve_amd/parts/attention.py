@@ -18,9 +18,9 @@ def tiled_attention(ops, q, q_stride, k_pages, v_pages, table, ctx, **rule) -> t
     tiles = None
     if ctx.num_prefill_seqs > 0:
         reach = (rule.get("window"), rule.get("chunk"))
-        tiles = ctx.derive(("attention_tiles_64", *reach), lambda step: torch.tensor(
+        tiles = ctx.derive(("attention_tiles_64", *reach), lambda step: ops.device_ints(
             ops.attention_tile_list(step.query_lens[:step.num_prefill_seqs], step.context_lens_host[:step.num_prefill_seqs],
-                                    window=reach[0], chunk=reach[1]), dtype=torch.int32, device=q.device))
+                                    window=reach[0], chunk=reach[1])))
     return ops.attention_tiles(
         q, q_stride, k_pages, v_pages, table, ctx.query_start_loc, ctx.context_lens, tokens=ctx.num_tokens,
         prefill_tiles=tiles, num_prefill_seqs=ctx.num_prefill_seqs, num_decode_seqs=ctx.num_decode_seqs,

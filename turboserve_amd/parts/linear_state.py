@@ -4,7 +4,6 @@ from __future__ import annotations
 
 from collections.abc import Mapping
 
-import numpy as np
 import torch
 
 from turboserve_amd.parts.base import CacheNeed, FixedState, FixedStateView, Mixer, Runtime, TensorSpec
@@ -126,5 +125,5 @@ class GatedLinearAttention(Mixer):
 
     def _plan(self, step, piece: int, device) -> tuple:
         pieces, carries = self.runtime.ops.linear_state_pieces(step.query_lens[: step.num_prefill_seqs], piece)
-        both = torch.from_numpy(np.asarray(pieces + carries, dtype=np.int32)).to(device)
+        both = self.runtime.ops.device_ints(pieces + carries)
         return both[: len(pieces)], both[len(pieces):], len(pieces), len(carries)
