@@ -428,6 +428,7 @@ extern "C" int ts_attention_tiles(void* out, void* partial_o, void* partial_ml, 
   if (dk < 8 || dk > 448 || dk % 8 != 0 || dv < 8 || dv > 384 || dv % 8 != 0 || block_size < 8 || block_size % 8 != 0)
     return TS_ERR_SHAPE;
   if (!v_pages && dv > dk) return TS_ERR_SHAPE;
+  if (block_size & (block_size - 1)) return TS_ERR_SHAPE;  // slots are taken apart by shift and mask
   if (v_pages && (dk > 384 || dv > 256)) return TS_ERR_SHAPE;  // the widest tiles are built for values inside the key rows
   if ((((uintptr_t)q | (uintptr_t)k_pages | (uintptr_t)v_pages) & 15) != 0 || (q_stride % 8) != 0) return TS_ERR_ARG;
   const FaRule rule = {scale, softcap, sinks, window, chunk};

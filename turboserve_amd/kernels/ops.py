@@ -1083,7 +1083,7 @@ class Ops:
         or a multiple of that."""
         widest = (448, 384) if values_in_keys else (384, 256)
         return (dtype == torch.bfloat16 and head_dim % 8 == 0 and 8 <= head_dim <= widest[0] and value_dim % 8 == 0
-                and 8 <= value_dim <= widest[1] and block_size % 8 == 0 and q_stride % 8 == 0)
+                and 8 <= value_dim <= widest[1] and block_size % 8 == 0 and block_size & (block_size - 1) == 0 and q_stride % 8 == 0)
 
     @staticmethod
     def attention_tile_list(query_lens, context_lens=None, rows: int = 64, *, window: int | None = None,
