@@ -98,7 +98,8 @@ template <typename T, typename P>
 __global__ void add_rmsnorm_kernel(T* __restrict__ y, float* __restrict__ residual,
                                    const P* __restrict__ pending, int splits, size_t split_stride,
                                    const T* __restrict__ w, const int* __restrict__ rows, float eps,
-                                   int hidden, float gain_offset, int one_rounding) {
+                                   int hidden, float gain_offset, int one_rounding,
+                                   const float* __restrict__ also, int also_splits, size_t also_stride) {
   __shared__ float scratch[16];
   const int src = rows ? rows[blockIdx.x] : blockIdx.x;
   const size_t in_base = (size_t)src * hidden;
@@ -106,10 +107,9 @@ __global__ void add_rmsnorm_kernel(T* __restrict__ y, float* __restrict__ residu
   float ss = 0.f;
   for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
     float s = residual[in_base + i];
-    if (pending) {
-      s = add_splits(pending + in_base + i, splits, split_stride, s);
-      if (!rows) residual[in_base + i] = s;  // re-read below by this same thread
-    }
+    if (pending) s = add_splits(pending + in_base + i, splits, split_stride, s);
+    if (also) s = add_splits(also + in_base + i, also_splits, also_stride, s);
+    if ((pending || also) && !rows) residual[in_base + i] = s;  // re-read below by this same thread
     ss += s * s;
   }
   ss = block_sum(ss, scratch);
@@ -117,6 +117,7 @@ __global__ void add_rmsnorm_kernel(T* __restrict__ y, float* __restrict__ residu
   for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
     float s = residual[in_base + i];
     if (rows && pending) s = add_splits(pending + in_base + i, splits, split_stride, s);
+    if (rows && also) s = add_splits(also + in_base + i, also_splits, also_stride, s);
     y[out_base + i] = from_float<T>(with_gain<T>(s * rstd, to_float(w[i]), gain_offset, one_rounding));
   }
 }
@@ -207,7 +208,8 @@ template <typename T, typename P>
 __global__ void add_rmsnorm_vec4_kernel(T* __restrict__ y, float* __restrict__ residual,
                                         const P* __restrict__ pending, int splits, size_t split_stride,
                                         const T* __restrict__ w, const int* __restrict__ rows, float eps,
-                                        int hidden, float gain_offset, int one_rounding) {
+                                        int hidden, float gain_offset, int one_rounding,
+                                        const float* __restrict__ also, int also_splits, size_t also_stride) {
   __shared__ float scratch[16];
   const int src = rows ? rows[blockIdx.x] : blockIdx.x;
   const size_t in_base = (size_t)src * hidden;
@@ -221,10 +223,9 @@ __global__ void add_rmsnorm_vec4_kernel(T* __restrict__ y, float* __restrict__ r
     if (qd < quads) {
       Vec4Of<float>::load(residual + in_base + 4 * qd, s[it]);
       Vec4Of<T>::load(w + 4 * qd, g[it]);  // with the other loads, not behind the reduction's barriers
-      if (pending) {
-        add_splits4(pending + in_base + 4 * qd, splits, split_stride, s[it]);
-        if (!rows) Vec4Of<float>::store(residual + in_base + 4 * qd, s[it]);
-      }
+      if (pending) add_splits4(pending + in_base + 4 * qd, splits, split_stride, s[it]);
+      if (also) add_splits4(also + in_base + 4 * qd, also_splits, also_stride, s[it]);
+      if ((pending || also) && !rows) Vec4Of<float>::store(residual + in_base + 4 * qd, s[it]);
 #pragma unroll
       for (int e = 0; e < 4; ++e) ss += s[it][e] * s[it][e];
     }
@@ -246,7 +247,8 @@ __global__ void add_rmsnorm_vec4_kernel(T* __restrict__ y, float* __restrict__ r
 template <typename T, typename P>
 static void launch_add_rmsnorm(void* y, float* residual, const void* pending, int splits, long split_stride,
                                const void* w, const int* rows, float eps, int out_rows, int hidden,
-                               float gain_offset, int one_rounding, hipStream_t stream) {
+                               float gain_offset, int one_rounding, const float* also, int also_splits,
+                               long also_stride, hipStream_t stream) {
   // Few rows (decode): one large block per row; many rows (prefill): just enough threads.
   int threads = out_rows <= 256 ? 1024 : 256;
   const int need = (hidden / 4 + NORM_ITEMS - 1) / NORM_ITEMS;
@@ -254,27 +256,30 @@ static void launch_add_rmsnorm(void* y, float* residual, const void* pending, in
   if (hidden % 4 == 0 && threads <= 1024) {
     hipLaunchKernelGGL((add_rmsnorm_vec4_kernel<T, P>), dim3(out_rows), dim3(threads), 0, stream, (T*)y, residual,
                        (const P*)pending, splits, (size_t)split_stride, (const T*)w, rows, eps, hidden, gain_offset,
-                       one_rounding);
+                       one_rounding, also, also_splits, (size_t)also_stride);
   } else {
     hipLaunchKernelGGL((add_rmsnorm_kernel<T, P>), dim3(out_rows), dim3(hidden <= 1024 ? 256 : 1024), 0, stream,
                        (T*)y, residual, (const P*)pending, splits, (size_t)split_stride, (const T*)w, rows, eps,
-                       hidden, gain_offset, one_rounding);
+                       hidden, gain_offset, one_rounding, also, also_splits, (size_t)also_stride);
   }
 }
 
 // `out_rows` = rows of y written: the number of entries of `rows` if given, else the tokens.
 // pending_f32 != 0: `pending` holds `splits` 32-bit partial sums, `split_stride` elements apart.
+// `also`: a second addend, `also_splits` 32-bit partial sums `also_stride` apart (a block whose two parts
+// both add to the stream), or null.
 extern "C" int ts_add_rmsnorm(void* y, float* residual, const void* pending, int pending_f32, int splits,
                               long split_stride, const void* w, const int* rows, float eps, int out_rows,
-                              int hidden, float gain_offset, int one_rounding, int dtype, hipStream_t stream) {
+                              int hidden, float gain_offset, int one_rounding, int dtype, const float* also,
+                              int also_splits, long also_stride, hipStream_t stream) {
   if (out_rows == 0) return TS_OK;
-  if (!y || !residual || !w || hidden < 1 || splits < 1) return TS_ERR_ARG;
+  if (!y || !residual || !w || hidden < 1 || splits < 1 || (also && also_splits < 1)) return TS_ERR_ARG;
   if (dtype == TS_F32)
-    launch_add_rmsnorm<float, float>(y, residual, pending, splits, split_stride, w, rows, eps, out_rows, hidden, gain_offset, one_rounding, stream);
+    launch_add_rmsnorm<float, float>(y, residual, pending, splits, split_stride, w, rows, eps, out_rows, hidden, gain_offset, one_rounding, also, also_splits, also_stride, stream);
   else if (dtype == TS_BF16 && pending_f32)
-    launch_add_rmsnorm<bf16_t, float>(y, residual, pending, splits, split_stride, w, rows, eps, out_rows, hidden, gain_offset, one_rounding, stream);
+    launch_add_rmsnorm<bf16_t, float>(y, residual, pending, splits, split_stride, w, rows, eps, out_rows, hidden, gain_offset, one_rounding, also, also_splits, also_stride, stream);
   else if (dtype == TS_BF16)
-    launch_add_rmsnorm<bf16_t, bf16_t>(y, residual, pending, splits, split_stride, w, rows, eps, out_rows, hidden, gain_offset, one_rounding, stream);
+    launch_add_rmsnorm<bf16_t, bf16_t>(y, residual, pending, splits, split_stride, w, rows, eps, out_rows, hidden, gain_offset, one_rounding, also, also_splits, also_stride, stream);
   else
     return TS_ERR_DTYPE;
   return ts_launch_status();

@@ -60,7 +60,7 @@ _SIGNATURES: dict[str, dict[str, list]] = {
         "ts_embed": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
         "ts_rmsnorm": [c_void_p, c_void_p, c_void_p, c_float, c_int, c_int, c_float, c_int, c_int, c_void_p],
         "ts_add_rmsnorm": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_void_p, c_void_p, c_float,
-                           c_int, c_int, c_float, c_int, c_int, c_void_p],
+                           c_int, c_int, c_float, c_int, c_int, c_void_p, c_int, c_long, c_void_p],
         "ts_swiglu": [c_void_p, c_void_p, c_int, c_int, c_long, c_int, c_int, c_int, c_float, c_float, c_float, c_float, c_int,
                       c_void_p],
         "ts_rope_store": [c_void_p, c_long, c_void_p, c_int, c_int, c_long, c_void_p, c_void_p, c_void_p, c_void_p,
@@ -420,11 +420,12 @@ class Ops:
         *,
         gain_offset: float = 0.0,
         one_rounding: bool = False,
+        also: torch.Tensor | None = None,
     ) -> torch.Tensor:
         """``residual += pending`` in 32-bit (in place) and the normalised sum in ``weight``'s
         dtype; with ``rows`` only those rows, and ``residual`` is left alone.  ``pending`` is a
-        ``[T, H]`` tensor of the run dtype or ``[S, T, H]`` 32-bit partial sums.  The gain is
-        applied as in :meth:`rmsnorm`."""
+        ``[T, H]`` tensor of the run dtype or ``[S, T, H]`` 32-bit partial sums.  ``also``: a second
+        addend, ``[S, T, H]`` 32-bit partial sums.  The gain is applied as in :meth:`rmsnorm`."""
         _gpu(residual, pending, weight, rows)
         _i32(rows, "rows")
         _need(residual.dim() == 2 and residual.dtype == torch.float32 and residual.is_contiguous(),
@@ -434,11 +435,18 @@ class Ops:
         is_f32, splits, stride = (0, 1, 0)
         if pending is not None:
             is_f32, splits, stride = self._partials(pending, tokens, hidden, weight.dtype, "pending")
+        also_splits, also_stride = 0, 0
+        if also is not None:
+            _gpu(also)
+            _need(also.dim() == 3 and also.dtype == torch.float32 and also.is_contiguous() and also.shape[1:] == (tokens, hidden),
+                  "a second addend must be float32 partial sums [S, T, H]")
+            also_splits, also_stride = also.shape[0], tokens * hidden
         out_rows = tokens if rows is None else rows.numel()
         y = self.rows_buffer(out_rows, hidden, weight.dtype, residual.device)
         _check(self.core.ts_add_rmsnorm(_ptr(y), _ptr(residual), _ptr(pending), is_f32, splits, stride, _ptr(weight),
                                         _ptr(rows), float(eps), out_rows, hidden, float(gain_offset),
-                                        1 if one_rounding else 0, dtype_code(weight.dtype), self.stream()),
+                                        1 if one_rounding else 0, dtype_code(weight.dtype), _ptr(also), also_splits,
+                                        also_stride, self.stream()),
                "ts_add_rmsnorm")
         return y
 

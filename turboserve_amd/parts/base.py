@@ -132,6 +132,9 @@ class ResidualStream:
 
     residual: torch.Tensor
     pending: torch.Tensor | None = None  # [T, H] run dtype, or [S, T, H] 32-bit partial sums
+    #: A second output that has not been added yet, ``[S, T, H]`` 32-bit partial sums: a block whose
+    #: two parts both add to the stream leaves one here, and the next norm adds both in its pass.
+    also: torch.Tensor | None = None
 
 
 # ---------------------------------------------------------------------------------------------

@@ -80,9 +80,10 @@ class PreNormBlock(Block):
 class ParallelBlock(Block):
     """``h += mixer(n) + feed_forward(n)`` with one ``n = norm(h)`` that both parts read.
 
-    The mixer's output is added into the 32-bit residual stream by a pass of its own
-    (``ops.stream_fold``); the feed-forward's waits in ``stream.pending`` for the next norm, as in
-    the pre-norm block.  A block without a feed-forward (``feed_forward=None``) leaves the mixer's
+    The feed-forward's output waits in ``stream.pending`` for the next norm, as in the pre-norm
+    block; the mixer's waits beside it in ``stream.also`` where it is 32-bit partial sums (steps of
+    few tokens), and is otherwise added into the 32-bit residual stream by a pass of its own
+    (``ops.stream_fold``).  A block without a feed-forward (``feed_forward=None``) leaves the mixer's
     output pending instead.  ``norm_name`` / ``mixer_name`` / ``ff_name`` are the checkpoint names
     of the parts under the block's prefix."""
 
@@ -129,6 +130,9 @@ class ParallelBlock(Block):
         if self.feed_forward is None:
             stream.pending = mixed
             return stream
-        self.runtime.ops.stream_fold(stream.residual, mixed, self.runtime.dtype)
+        if mixed.dim() == 3:  # 32-bit partial sums (steps of few tokens): the next norm adds them with the feed-forward's
+            stream.also = mixed
+        else:
+            self.runtime.ops.stream_fold(stream.residual, mixed, self.runtime.dtype)
         stream.pending = self.feed_forward.forward(x, ctx)
         return stream

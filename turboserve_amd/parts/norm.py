@@ -47,7 +47,7 @@ class RMSNorm(Norm):
 
     def forward_residual(self, stream: ResidualStream, rows: torch.Tensor | None = None) -> torch.Tensor:
         y = self.runtime.ops.add_rmsnorm(stream.residual, stream.pending, self.weight, self.eps, rows,
-                                         gain_offset=self.gain_offset, one_rounding=self.one_rounding)
+                                         gain_offset=self.gain_offset, one_rounding=self.one_rounding, also=stream.also)
         if rows is None:
-            stream.pending = None
+            stream.pending = stream.also = None
         return y

@@ -67,9 +67,10 @@ class OriginMix(StreamStep):
         if origin is None:
             raise ValueError(f"{self.prefix}: the step needs the embedding's output and was not given it")
         ops, dtype = self.runtime.ops, self.runtime.dtype
-        if stream.pending is not None:
-            ops.stream_fold(stream.residual, stream.pending, dtype)
-            stream.pending = None
+        for waiting in (stream.pending, stream.also):
+            if waiting is not None:
+                ops.stream_fold(stream.residual, waiting, dtype)
+        stream.pending = stream.also = None
         mixed = ops.linear(ops.stream_pair(stream.residual, origin, dtype), self.weight, for_residual=True)
         ops.stream_fold(stream.residual, mixed, dtype, assign=True)
         return stream
